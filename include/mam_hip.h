@@ -1,0 +1,125 @@
+/*
+ * mam_hip.h -- C ABI of libmam_hip.so: the Multiply-And-Max/min (MAM) fully-connected
+ * hot path as hand-written HIP kernels for gfx950 (MI355X, wave64).
+ *
+ * Plain pointers and sizes only; every pointer is DEVICE memory of the current HIP
+ * device unless stated otherwise; `stream` is a hipStream_t passed as void* (NULL = the
+ * legacy default stream).  All calls are asynchronous on `stream`, never synchronise the
+ * host, and allocate nothing: scratch memory is brought in by the caller as `workspace`.
+ * Every function returns MAM_OK (0) or a negative MAM_ERR_* code; mam_error_string()
+ * names a code and mam_last_error() gives the detail of this thread's last failure.
+ *
+ * Notation: N = batch rows, K = in_features, M = out_features.
+ *   x        (N, K) fp32, row stride ldx (>= K)
+ *   w        layout MAM_W_KM: (K, M) fp32, row stride ldw (>= M) -- operand `b` of the
+ *            reference operators; layout MAM_W_MK: (M, K) fp32, row stride ldw (>= K) --
+ *            the nn.Module's `weight` (out, in), so the module needs no transposed copy.
+ *   c        (N, M) fp32 contiguous;   argmax/argmin (N, M) int32 contiguous.
+ *
+ * Each entry point names the interface of SSIGPRO/mamtorch 1.5.2 that it stands behind.
+ */
+#ifndef MAM_HIP_H
+#define MAM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MAM_OK 0
+#define MAM_ERR_INVALID_ARGUMENT (-1) /* null pointer, negative size, bad enum          */
+#define MAM_ERR_UNSUPPORTED (-2)      /* size outside what the kernels cover            */
+#define MAM_ERR_WORKSPACE (-3)        /* workspace missing or smaller than required     */
+#define MAM_ERR_LAUNCH (-4)           /* HIP reported an error at launch                */
+
+#define MAM_W_KM 0
+#define MAM_W_MK 1
+
+#define MAM_COUNT_REFERENCE 0 /* per call: +1 per (m,k) picked as max by >=1 row, +1 if picked as
+                                 min by >=1 row, both into max_count (the module's literal rule) */
+#define MAM_COUNT_HITS 1      /* true hit counts: max_count += #argmax hits, min_count += #argmin */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int mam_version(void);
+const char *mam_error_string(int code);
+const char *mam_last_error(void);
+
+/*
+ * Exact MAM forward with indices.
+ *   c[n,m]      = (max_k x[n,k]*w[k,m] + min_k x[n,k]*w[k,m]) (+ bias[m] if bias != NULL)
+ *   argmax[n,m] = lowest k attaining the max; argmin[n,m] = lowest k attaining the min.
+ * Replaces mamtorch_kernel_v1::fullyconnected_cuda
+ * (mamtorch/kernel/v1/csrc/cuda/fullyconnected.cu:177-291, kernel :33-175) and serves
+ * mamtorch_kernel_v4::fullyconnected_cuda (mamtorch/kernel/v4/csrc/cuda/fullyconnected.cu:41-149)
+ * with zero approximation error; the bias add is nn/v4/fullyconnected.py:197-198.
+ * NaN products are ignored, as by the reference kernel's ordered comparisons.
+ * `workspace` may be NULL when mam_fc_forward_workspace() returns 0.
+ */
+size_t mam_fc_forward_workspace(int64_t N, int64_t K, int64_t M);
+int mam_fc_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                   const float *bias, float *c, int32_t *argmax, int32_t *argmin,
+                   int64_t N, int64_t K, int64_t M,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Values-only exact forward (no indices).  Replaces mamtorch_kernel_v4::fullyconnected_fast_cuda
+ * (mamtorch/kernel/v4/csrc/cuda/fullyconnected_fast.cu:39-137, kernel
+ * fullyconnected_fast_kernel.cu:29-161).  Same c as mam_fc_forward, bit for bit.
+ */
+size_t mam_fc_forward_values_workspace(int64_t N, int64_t K, int64_t M);
+int mam_fc_forward_values(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                          const float *bias, float *c, int64_t N, int64_t K, int64_t M,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * MAM backward: routes grad only through the selected positions.
+ *   x_grad[n,k] = sum_m grad[n,m] * w[k,m] * ([k==argmax[n,m]] + [k==argmin[n,m]])
+ *   w_grad[k,m] = sum_n grad[n,m] * x[n,k] * (same)          (argmax==argmin counts twice)
+ * x_grad (N,K) and w_grad (layout and shape of w, contiguous) are fully overwritten.
+ * Either output pointer may be NULL to skip it.  grad/argmax/argmin are (N,M) contiguous.
+ * Replaces fullyconnected_backward_cuda
+ * (mamtorch/kernel/v4/csrc/cuda/fullyconnected_backward.cu:80-135, kernel :24-78; v1 identical).
+ * Indices outside [0,K) make the call's result undefined for that output only (they are skipped).
+ */
+int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                    const float *grad, const int32_t *argmax, const int32_t *argmin,
+                    float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, void *stream);
+
+/*
+ * Selection-count accumulation for pruning: adds this batch's picks into (M,K) int32 counters
+ * in place.  Replaces FullyConnected.update_selection_count
+ * (mamtorch/nn/v4/fullyconnected.py:114-129).  min_count may be NULL in MAM_COUNT_REFERENCE mode.
+ */
+int mam_selection_count(const int32_t *argmax, const int32_t *argmin, int32_t *max_count,
+                        int32_t *min_count, int64_t N, int64_t M, int64_t K, int mode, void *stream);
+
+/*
+ * CSR-sparse MAM forward over a pruned weight (M,K): CSR row m = output neuron m,
+ * crow (M+1) / col (nnz) int64, val (nnz) fp32, column indices strictly ascending within a
+ * row -- the operand convention of mamtorch_kernel_sparsev1::cusparsemm_csr
+ * (mamtorch/sparse/kernel/v1/csrc/cuda/cusparsemm_csr.cu:25-45).  The result equals
+ * mam_fc_forward on the densified weight: absent entries are zeros that take part in the
+ * max/min and in the first-index tie-break.  The reference has no sparse MAM operator.
+ */
+size_t mam_csr_fc_forward_workspace(int64_t N, int64_t K, int64_t M);
+int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
+                       const float *val, const float *bias, float *c, int32_t *argmax,
+                       int32_t *argmin, int64_t N, int64_t K, int64_t M,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * CSR-sparse MAM backward: x_grad (N,K) dense and val_grad (nnz), both fully overwritten.
+ * A selected column that is not stored in its row (an implicit zero won) has no weight
+ * gradient and adds nothing to x_grad.
+ */
+int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
+                        const float *val, const float *grad, const int32_t *argmax,
+                        const int32_t *argmin, float *x_grad, float *val_grad,
+                        int64_t N, int64_t K, int64_t M, int64_t nnz, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAM_HIP_H */

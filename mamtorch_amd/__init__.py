@@ -1,0 +1,16 @@
+"""MI355X-native Multiply-And-Max/min (MAM) fully-connected hot path.
+
+Mirrors the interface of SSIGPRO/mamtorch for this path (mamtorch/__init__.py:1-3):
+``kernel`` (operator wrappers), ``nn`` (FullyConnected), ``sparse`` (CSR-sparse MAM), plus
+``capi`` (the C ABI through ctypes).
+"""
+from . import _native
+
+_native.load_ops()
+
+from . import kernel  # noqa: E402
+from . import nn  # noqa: E402
+from . import sparse  # noqa: E402
+from . import capi  # noqa: E402
+
+__version__ = "0.1.0"

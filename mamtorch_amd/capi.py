@@ -1,0 +1,164 @@
+"""The C ABI of libmam_hip.so (include/mam_hip.h) through ctypes, for torch GPU tensors.
+
+Thin argument marshalling only: device pointers come from ``Tensor.data_ptr()``, the stream from
+``torch.cuda.current_stream()``, outputs and workspace from torch's allocator.  This is the path
+the GPU parity tests drive, and what a non-PyTorch host would bind.
+"""
+import ctypes
+
+import torch
+
+from . import _native
+
+W_KM = 0
+W_MK = 1
+COUNT_REFERENCE = 0
+COUNT_HITS = 1
+
+EXPORTS = (
+    "mam_version", "mam_error_string", "mam_last_error",
+    "mam_fc_forward_workspace", "mam_fc_forward",
+    "mam_fc_forward_values_workspace", "mam_fc_forward_values",
+    "mam_fc_backward", "mam_selection_count",
+    "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward",
+)
+
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_ptr = ctypes.c_void_p
+_size = ctypes.c_size_t
+_configured = False
+
+
+def lib():
+    global _configured
+    l = _native.hip_library()
+    if not _configured:
+        l.mam_error_string.restype = ctypes.c_char_p
+        l.mam_error_string.argtypes = [_int]
+        l.mam_last_error.restype = ctypes.c_char_p
+        for name in ("mam_fc_forward_workspace", "mam_fc_forward_values_workspace",
+                     "mam_csr_fc_forward_workspace"):
+            fn = getattr(l, name)
+            fn.restype = _size
+            fn.argtypes = [_i64, _i64, _i64]
+        l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64,
+                                     _ptr, _size, _ptr]
+        l.mam_fc_forward_values.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _i64, _i64, _i64,
+                                            _ptr, _size, _ptr]
+        l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
+                                      _i64, _ptr]
+        l.mam_selection_count.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr]
+        l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
+                                         _i64, _ptr, _size, _ptr]
+        l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
+                                          _i64, _i64, _i64, _ptr]
+        _configured = True
+    return l
+
+
+class MamError(RuntimeError):
+    def __init__(self, code):
+        self.code = code
+        l = lib()
+        super().__init__("%s (%s)" % (l.mam_error_string(code).decode(), l.mam_last_error().decode()))
+
+
+def _check(rc):
+    if rc != 0:
+        raise MamError(rc)
+
+
+def _p(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _dims(x, w, layout):
+    N, K = x.shape
+    M = w.shape[0] if layout == W_MK else w.shape[1]
+    return N, K, M
+
+
+def _ld(t):
+    return t.stride(0) if t.size(0) > 1 else max(t.size(1), 1)
+
+
+def fc_forward(x, w, layout=W_KM, bias=None, workspace=None):
+    """-> (c, argmax, argmin) on x.device.  ``workspace`` (uint8 tensor) is allocated if None."""
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    c = torch.empty((N, M), dtype=torch.float32, device=x.device)
+    amax = torch.empty((N, M), dtype=torch.int32, device=x.device)
+    amin = torch.empty((N, M), dtype=torch.int32, device=x.device)
+    need = l.mam_fc_forward_workspace(N, K, M)
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(l.mam_fc_forward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(bias), _p(c), _p(amax), _p(amin),
+                                N, K, M, _p(workspace), 0 if workspace is None else workspace.numel(),
+                                _stream(x)))
+    return c, amax, amin
+
+
+def fc_forward_values(x, w, layout=W_KM, bias=None, workspace=None):
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    c = torch.empty((N, M), dtype=torch.float32, device=x.device)
+    need = l.mam_fc_forward_values_workspace(N, K, M)
+    if workspace is None and need:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(l.mam_fc_forward_values(_p(x), _ld(x), _p(w), _ld(w), layout, _p(bias), _p(c), N, K, M,
+                                       _p(workspace), 0 if workspace is None else workspace.numel(),
+                                       _stream(x)))
+    return c
+
+
+def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=True):
+    """-> (x_grad or None, w_grad or None); w_grad has the shape and layout of w."""
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    xg = torch.empty((N, K), dtype=torch.float32, device=x.device) if want_x else None
+    wg = torch.empty(tuple(w.shape), dtype=torch.float32, device=x.device) if want_w else None
+    with torch.cuda.device(x.device):
+        _check(l.mam_fc_backward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(grad), _p(argmax), _p(argmin),
+                                 _p(xg), _p(wg), N, K, M, _stream(x)))
+    return xg, wg
+
+
+def selection_count(argmax, argmin, max_count, min_count, mode=COUNT_REFERENCE):
+    """In place on the (M, K) int32 counters."""
+    l = lib()
+    N, M = argmax.shape
+    K = max_count.shape[1]
+    with torch.cuda.device(argmax.device):
+        _check(l.mam_selection_count(_p(argmax), _p(argmin), _p(max_count), _p(min_count), N, M, K, mode,
+                                     _stream(argmax)))
+
+
+def csr_fc_forward(x, crow, col, val, M, bias=None):
+    l = lib()
+    N, K = x.shape
+    c = torch.empty((N, M), dtype=torch.float32, device=x.device)
+    amax = torch.empty((N, M), dtype=torch.int32, device=x.device)
+    amin = torch.empty((N, M), dtype=torch.int32, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(l.mam_csr_fc_forward(_p(x), _ld(x), _p(crow), _p(col), _p(val), _p(bias), _p(c), _p(amax),
+                                    _p(amin), N, K, M, None, 0, _stream(x)))
+    return c, amax, amin
+
+
+def csr_fc_backward(x, crow, col, val, grad, argmax, argmin):
+    l = lib()
+    N, K = x.shape
+    M = crow.numel() - 1
+    xg = torch.empty((N, K), dtype=torch.float32, device=x.device)
+    vg = torch.empty_like(val)
+    with torch.cuda.device(x.device):
+        _check(l.mam_csr_fc_backward(_p(x), _ld(x), _p(crow), _p(col), _p(val), _p(grad), _p(argmax),
+                                     _p(argmin), _p(xg), _p(vg), N, K, M, val.numel(), _stream(x)))
+    return xg, vg

@@ -1,0 +1,456 @@
+// Exact MAM forward for gfx950 (MI355X): c = max_k(x*w) + min_k(x*w) (+ bias), with the
+// lowest k attaining each extreme.  Replaces the reference's v1 exact kernel
+// (mamtorch/kernel/v1/csrc/cuda/fullyconnected.cu:33-175), serves the v4 operator, and the
+// values-only variant replaces v4's fullyconnected_fast kernel
+// (mamtorch/kernel/v4/csrc/cuda/fullyconnected_fast_kernel.cu:29-161).
+//
+// The (max, min, x) semiring has no matrix-core form, so the kernel is FP32-VALU bound and
+// is organised to spend as few VALU issue slots per product as possible:
+//
+//   * One v_mul_f32 per product; v_max3_f32 / v_min3_f32 fold TWO products into the
+//     running extreme per issue slot.  That is 2 slots per (multiply, max, min) triple.
+//   * Indices are NOT tracked per product.  Products are consumed in groups of G = 8
+//     consecutive k; after a group, one compare + one select per extreme records the group
+//     id if the running extreme strictly improved (0.5 slot per triple).  Because the test is
+//     strict, the recorded group is the one holding the FIRST occurrence of the final extreme.
+//   * An epilogue re-reads the 8 operands of the recorded group, finds the first k whose
+//     product equals the extreme, and recomputes the value from that k.  Recomputing also
+//     removes the +0/-0 ambiguity of the hardware max/min, so values and indices are exactly
+//     those of a scalar scan in ascending k with strict comparisons.
+//
+// Tiling: a workgroup of 256 threads (4 waves, one per SIMD) owns a 64 x 128 tile of c.  X and
+// W tiles of 32 consecutive k are staged in LDS as [row][k] (row stride 36 floats: 16-byte
+// aligned and conflict-free for ds_read_b128 along k).  A thread owns 4 x 8 outputs, strided
+// by 16 in both directions, so that a wave's W reads cover all banks and its X reads
+// broadcast.  128 of its registers hold (max, min, group-of-max, group-of-min); two
+// workgroups share a CU, so each SIMD always has a second wave to issue from while the other
+// waits on LDS or on the tile barrier.  Ragged edges are handled by replicating the last row /
+// column / k on load: a replicated k duplicates an earlier product and can never win a
+// strict comparison.
+//
+// Small N*M (the 256 x 4096 headline shape has only 512 tiles for 256 CUs x 2) is split
+// along K; each split writes (value, group) partials and a merge kernel combines them in
+// ascending k order with the same strict comparisons before resolving indices.
+#include "mam_common.h"
+
+namespace mam {
+namespace fwd {
+
+constexpr int BN = 64;        // batch rows per workgroup
+constexpr int BM = 128;       // output neurons per workgroup
+constexpr int KT = 32;        // k extent of one LDS tile
+constexpr int LDK = KT + 4;   // LDS row stride in floats
+constexpr int G = 8;          // products per index-tracking group
+constexpr int TI = 4;         // rows per thread
+constexpr int TJ = 8;         // columns per thread
+constexpr int NT = 256;       // threads per workgroup
+constexpr int GROUP_N = 8;    // row tiles swept together so that W panels are reused from L2
+constexpr int MAX_SPLITS = 8;
+
+struct Params {
+    const float *x;
+    int64_t ldx;
+    const float *w;
+    int64_t ldw;
+    const float *bias;
+    float *c;
+    int32_t *argmax;
+    int32_t *argmin;
+    float *part;      // split-K partials: [split][4 or 2][N*M]
+    int N, K, M;
+    int tiles_n, tiles_m, splits, k_per_split;
+    int vec_x, vec_w;  // 16-byte global loads are legal for x / w
+};
+
+// First k in group g (ascending) whose product equals `target`; value recomputed from it.
+template <int LAYOUT>
+__device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, float target,
+                                        float &val, int &idx)
+{
+    const int kb = g * G;
+    const int klast = p.K - 1;
+    idx = kb < klast ? kb : klast;
+    val = target;
+    const float *xr = p.x + (int64_t)n * p.ldx;
+#pragma unroll
+    for (int kk = G - 1; kk >= 0; --kk) {
+        const int k = (kb + kk) < klast ? (kb + kk) : klast;
+        const float prod = xr[k] * load_w<LAYOUT>(p.w, p.ldw, k, m);
+        if (prod == target) { idx = k; val = prod; }
+    }
+}
+
+// A zero extreme carries the sign of the FIRST zero product; the hardware max/min may have
+// kept another zero's sign.  Rare (whole column of products has no positive / no negative
+// entry), so a plain scan is enough.
+template <int LAYOUT>
+__device__ __noinline__ float first_zero_product(const Params &p, int n, int m)
+{
+    const float *xr = p.x + (int64_t)n * p.ldx;
+    for (int k = 0; k < p.K; ++k) {
+        const float prod = xr[k] * load_w<LAYOUT>(p.w, p.ldw, k, m);
+        if (prod == 0.0f) return prod;
+    }
+    return 0.0f;
+}
+
+template <int LAYOUT, bool ARGS>
+__device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax, float vmin,
+                                       int gmax, int gmin)
+{
+    float hi = vmax, lo = vmin;
+    int ih = 0, il = 0;
+    if (ARGS) {
+        resolve<LAYOUT>(p, n, m, gmax, vmax, hi, ih);
+        resolve<LAYOUT>(p, n, m, gmin, vmin, lo, il);
+    } else {
+        if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m);
+        if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m);
+    }
+    float s = hi + lo;
+    if (p.bias) s = s + p.bias[m];
+    const int64_t o = (int64_t)n * p.M + m;
+    p.c[o] = s;
+    if (ARGS) {
+        p.argmax[o] = ih;
+        p.argmin[o] = il;
+    }
+}
+
+template <int LAYOUT, bool ARGS>
+__global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
+{
+    __shared__ __attribute__((aligned(16))) float xs[BN][LDK];
+    __shared__ __attribute__((aligned(16))) float ws[BM][LDK];
+
+    const int tid = threadIdx.x;
+    const int tx = tid & 15;  // column lane: columns tx + 16*j
+    const int ty = tid >> 4;  // row lane:    rows    ty + 16*i
+
+    // ---- which tile: XCD-aware, then row tiles grouped under one W panel ----
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int tiles = p.tiles_n * p.tiles_m;
+    const int split = logical / tiles;
+    const int l = logical - split * tiles;
+    const int per_group = GROUP_N * p.tiles_m;
+    const int grp = l / per_group;
+    const int first_n = grp * GROUP_N;
+    const int gsize = (p.tiles_n - first_n) < GROUP_N ? (p.tiles_n - first_n) : GROUP_N;
+    const int lin = l - grp * per_group;
+    const int tn = first_n + lin % gsize;
+    const int tm = lin / gsize;
+    const int row0 = tn * BN, col0 = tm * BM;
+    const int kb = split * p.k_per_split;
+    const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
+
+    float vmax[TI][TJ], vmin[TI][TJ];
+    int gmax[TI][TJ], gmin[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            vmax[i][j] = -__builtin_inff();
+            vmin[i][j] = __builtin_inff();
+            gmax[i][j] = kb / G;
+            gmin[i][j] = kb / G;
+        }
+
+    for (int k0 = kb; k0 < ke; k0 += KT) {
+        // ---- stage the X tile: 64 rows x 8 chunks of 4 k ----
+        float4 xr[(BN * KT / 4) / NT];
+#pragma unroll
+        for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
+            const int e = tid + it * NT;
+            const int r = e >> 3, ch = e & 7;
+            const int row = (row0 + r) < p.N ? (row0 + r) : (p.N - 1);
+            const int k = k0 + ch * 4;
+            const float *src = p.x + (int64_t)row * p.ldx;
+            if (p.vec_x && k + 3 < ke) {
+                xr[it] = *reinterpret_cast<const float4 *>(src + k);
+            } else {
+                const int kl = ke - 1;
+                xr[it].x = src[k < kl ? k : kl];
+                xr[it].y = src[k + 1 < kl ? k + 1 : kl];
+                xr[it].z = src[k + 2 < kl ? k + 2 : kl];
+                xr[it].w = src[k + 3 < kl ? k + 3 : kl];
+            }
+        }
+        // ---- stage the W tile ----
+        float4 wr[(BM * KT / 4) / NT];
+        if (LAYOUT == MAM_W_MK) {
+#pragma unroll
+            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+                const int e = tid + it * NT;
+                const int r = e >> 3, ch = e & 7;
+                const int col = (col0 + r) < p.M ? (col0 + r) : (p.M - 1);
+                const int k = k0 + ch * 4;
+                const float *src = p.w + (int64_t)col * p.ldw;
+                if (p.vec_w && k + 3 < ke) {
+                    wr[it] = *reinterpret_cast<const float4 *>(src + k);
+                } else {
+                    const int kl = ke - 1;
+                    wr[it].x = src[k < kl ? k : kl];
+                    wr[it].y = src[k + 1 < kl ? k + 1 : kl];
+                    wr[it].z = src[k + 2 < kl ? k + 2 : kl];
+                    wr[it].w = src[k + 3 < kl ? k + 3 : kl];
+                }
+            }
+        } else {
+            // (K, M) operand: rows of w are contiguous along m; 8 lanes fetch 128 bytes of
+            // one k, and the tile is transposed on the way into LDS.
+#pragma unroll
+            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+                const int e = tid + it * NT;
+                const int c4 = (e & 7) + ((e >> 8) << 3);
+                const int kk = (e >> 3) & 31;
+                const int k = (k0 + kk) < ke ? (k0 + kk) : (ke - 1);
+                const int mb = col0 + c4 * 4;
+                const float *src = p.w + (int64_t)k * p.ldw;
+                if (p.vec_w && mb + 3 < p.M) {
+                    wr[it] = *reinterpret_cast<const float4 *>(src + mb);
+                } else {
+                    const int ml = p.M - 1;
+                    wr[it].x = src[mb < ml ? mb : ml];
+                    wr[it].y = src[mb + 1 < ml ? mb + 1 : ml];
+                    wr[it].z = src[mb + 2 < ml ? mb + 2 : ml];
+                    wr[it].w = src[mb + 3 < ml ? mb + 3 : ml];
+                }
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
+            const int e = tid + it * NT;
+            *reinterpret_cast<float4 *>(&xs[e >> 3][(e & 7) * 4]) = xr[it];
+        }
+        if (LAYOUT == MAM_W_MK) {
+#pragma unroll
+            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+                const int e = tid + it * NT;
+                *reinterpret_cast<float4 *>(&ws[e >> 3][(e & 7) * 4]) = wr[it];
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+                const int e = tid + it * NT;
+                const int c4 = (e & 7) + ((e >> 8) << 3);
+                const int kk = (e >> 3) & 31;
+                ws[c4 * 4 + 0][kk] = wr[it].x;
+                ws[c4 * 4 + 1][kk] = wr[it].y;
+                ws[c4 * 4 + 2][kk] = wr[it].z;
+                ws[c4 * 4 + 3][kk] = wr[it].w;
+            }
+        }
+        __syncthreads();
+
+        // ---- 4 groups of 8 k: 32 outputs x 8 products each ----
+#pragma unroll 2
+        for (int gg = 0; gg < KT / G; ++gg) {
+            const int g = k0 / G + gg;
+            float4 xv[TI][2];
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                xv[i][0] = *reinterpret_cast<const float4 *>(&xs[ty + 16 * i][gg * G]);
+                xv[i][1] = *reinterpret_cast<const float4 *>(&xs[ty + 16 * i][gg * G + 4]);
+            }
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                const float4 wa = *reinterpret_cast<const float4 *>(&ws[tx + 16 * j][gg * G]);
+                const float4 wb = *reinterpret_cast<const float4 *>(&ws[tx + 16 * j][gg * G + 4]);
+#pragma unroll
+                for (int i = 0; i < TI; ++i) {
+                    const float p0 = xv[i][0].x * wa.x, p1 = xv[i][0].y * wa.y;
+                    const float p2 = xv[i][0].z * wa.z, p3 = xv[i][0].w * wa.w;
+                    const float p4 = xv[i][1].x * wb.x, p5 = xv[i][1].y * wb.y;
+                    const float p6 = xv[i][1].z * wb.z, p7 = xv[i][1].w * wb.w;
+                    const float om = vmax[i][j];
+                    float hi = __builtin_fmaxf(__builtin_fmaxf(om, p0), p1);
+                    hi = __builtin_fmaxf(__builtin_fmaxf(hi, p2), p3);
+                    hi = __builtin_fmaxf(__builtin_fmaxf(hi, p4), p5);
+                    hi = __builtin_fmaxf(__builtin_fmaxf(hi, p6), p7);
+                    const float on = vmin[i][j];
+                    float lo = __builtin_fminf(__builtin_fminf(on, p0), p1);
+                    lo = __builtin_fminf(__builtin_fminf(lo, p2), p3);
+                    lo = __builtin_fminf(__builtin_fminf(lo, p4), p5);
+                    lo = __builtin_fminf(__builtin_fminf(lo, p6), p7);
+                    if (ARGS) {
+                        gmax[i][j] = (hi > om) ? g : gmax[i][j];
+                        gmin[i][j] = (lo < on) ? g : gmin[i][j];
+                    }
+                    vmax[i][j] = hi;
+                    vmin[i][j] = lo;
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue ----
+    if (p.splits == 1) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                const int n = row0 + ty + 16 * i, m = col0 + tx + 16 * j;
+                if (n < p.N && m < p.M)
+                    finish<LAYOUT, ARGS>(p, n, m, vmax[i][j], vmin[i][j], gmax[i][j], gmin[i][j]);
+            }
+    } else {
+        const int64_t nm = (int64_t)p.N * p.M;
+        float *base = p.part + (int64_t)split * (ARGS ? 4 : 2) * nm;
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                const int n = row0 + ty + 16 * i, m = col0 + tx + 16 * j;
+                if (n < p.N && m < p.M) {
+                    const int64_t o = (int64_t)n * p.M + m;
+                    base[o] = vmax[i][j];
+                    base[nm + o] = vmin[i][j];
+                    if (ARGS) {
+                        base[2 * nm + o] = __int_as_float(gmax[i][j]);
+                        base[3 * nm + o] = __int_as_float(gmin[i][j]);
+                    }
+                }
+            }
+    }
+}
+
+// Combines split-K partials in ascending k order (strict comparisons keep the earliest
+// group on ties), then resolves indices / zero signs exactly as the single-pass epilogue.
+template <int LAYOUT, bool ARGS>
+__global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
+{
+    const int64_t nm = (int64_t)p.N * p.M;
+    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (o >= nm) return;
+    const int stride = ARGS ? 4 : 2;
+    float vmax = p.part[o], vmin = p.part[nm + o];
+    int gmax = 0, gmin = 0;
+    if (ARGS) {
+        gmax = __float_as_int(p.part[2 * nm + o]);
+        gmin = __float_as_int(p.part[3 * nm + o]);
+    }
+    for (int s = 1; s < p.splits; ++s) {
+        const float *base = p.part + (int64_t)s * stride * nm;
+        const float hi = base[o], lo = base[nm + o];
+        if (hi > vmax) {
+            vmax = hi;
+            if (ARGS) gmax = __float_as_int(base[2 * nm + o]);
+        }
+        if (lo < vmin) {
+            vmin = lo;
+            if (ARGS) gmin = __float_as_int(base[3 * nm + o]);
+        }
+    }
+    const int n = (int)(o / p.M), m = (int)(o - (int64_t)n * p.M);
+    finish<LAYOUT, ARGS>(p, n, m, vmax, vmin, gmax, gmin);
+}
+
+// How many K ranges to split into so that at least two workgroups reach every CU.
+static int choose_splits(int64_t N, int64_t K, int64_t M)
+{
+    const int64_t tiles = ceil_div(N, BN) * ceil_div(M, BM);
+    const int64_t want = 2 * kNumCU;
+    if (tiles >= want) return 1;
+    int64_t s = ceil_div(want, tiles);
+    const int64_t max_by_k = K / (8 * KT);  // keep at least 256 k per split
+    if (s > max_by_k) s = max_by_k;
+    if (s > MAX_SPLITS) s = MAX_SPLITS;
+    return s < 1 ? 1 : (int)s;
+}
+
+static size_t workspace_bytes(int64_t N, int64_t K, int64_t M, bool args)
+{
+    const int s = choose_splits(N, K, M);
+    if (s == 1) return 0;
+    return (size_t)s * (args ? 4 : 2) * (size_t)N * (size_t)M * sizeof(float);
+}
+
+template <bool ARGS>
+static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                  const float *bias, float *c, int32_t *argmax, int32_t *argmin, int64_t N,
+                  int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream)
+{
+    if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
+    if (w_layout != MAM_W_KM && w_layout != MAM_W_MK)
+        return fail(MAM_ERR_INVALID_ARGUMENT, "w_layout must be MAM_W_KM or MAM_W_MK");
+    if (N == 0 || M == 0) return MAM_OK;
+    if (K == 0) return fail(MAM_ERR_INVALID_ARGUMENT, "K == 0: max/min over an empty set");
+    if (!x || !w || !c || (ARGS && (!argmax || !argmin)))
+        return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    if (ldx < K || ldw < (w_layout == MAM_W_MK ? K : M))
+        return fail(MAM_ERR_INVALID_ARGUMENT, "leading dimension smaller than the row length");
+    if (N > INT32_MAX / 2 || K > INT32_MAX / 2 || M > INT32_MAX / 2)
+        return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
+
+    Params p;
+    p.x = x; p.ldx = ldx; p.w = w; p.ldw = ldw; p.bias = bias;
+    p.c = c; p.argmax = argmax; p.argmin = argmin;
+    p.N = (int)N; p.K = (int)K; p.M = (int)M;
+    p.tiles_n = (int)ceil_div(N, BN);
+    p.tiles_m = (int)ceil_div(M, BM);
+    p.splits = choose_splits(N, K, M);
+    p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), KT) * KT);
+    p.splits = (int)ceil_div(K, p.k_per_split);
+    p.part = nullptr;
+    if (p.splits > 1) {
+        const size_t need = (size_t)p.splits * (ARGS ? 4 : 2) * (size_t)N * (size_t)M * sizeof(float);
+        if (!workspace || workspace_size < need)
+            return fail(MAM_ERR_WORKSPACE, "forward needs %zu workspace bytes, got %zu", need,
+                        workspace ? workspace_size : (size_t)0);
+        p.part = static_cast<float *>(workspace);
+    }
+    p.vec_x = (ldx % 4 == 0) && ((uintptr_t)x % 16 == 0);
+    p.vec_w = (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0);
+
+    const int64_t nblk = (int64_t)p.tiles_n * p.tiles_m * p.splits;
+    if (nblk > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "too many tiles");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (w_layout == MAM_W_MK)
+        hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_MK, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
+    else
+        hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_KM, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
+    int rc = check_launch("mam_fwd_kernel");
+    if (rc != MAM_OK) return rc;
+    if (p.splits > 1) {
+        const unsigned mb = (unsigned)ceil_div(N * M, 256);
+        if (w_layout == MAM_W_MK)
+            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS>), dim3(mb), dim3(256), 0, st, p);
+        else
+            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_KM, ARGS>), dim3(mb), dim3(256), 0, st, p);
+        rc = check_launch("mam_fwd_merge_kernel");
+    }
+    return rc;
+}
+
+}  // namespace fwd
+}  // namespace mam
+
+extern "C" size_t mam_fc_forward_workspace(int64_t N, int64_t K, int64_t M)
+{
+    if (N <= 0 || K <= 0 || M <= 0) return 0;
+    return mam::fwd::workspace_bytes(N, K, M, true);
+}
+
+extern "C" size_t mam_fc_forward_values_workspace(int64_t N, int64_t K, int64_t M)
+{
+    if (N <= 0 || K <= 0 || M <= 0) return 0;
+    return mam::fwd::workspace_bytes(N, K, M, false);
+}
+
+extern "C" int mam_fc_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                              const float *bias, float *c, int32_t *argmax, int32_t *argmin,
+                              int64_t N, int64_t K, int64_t M, void *workspace,
+                              size_t workspace_bytes, void *stream)
+{
+    return mam::fwd::launch<true>(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, N, K, M,
+                                  workspace, workspace_bytes, stream);
+}
+
+extern "C" int mam_fc_forward_values(const float *x, int64_t ldx, const float *w, int64_t ldw,
+                                     int w_layout, const float *bias, float *c, int64_t N, int64_t K,
+                                     int64_t M, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return mam::fwd::launch<false>(x, ldx, w, ldw, w_layout, bias, c, nullptr, nullptr, N, K, M,
+                                   workspace, workspace_bytes, stream);
+}

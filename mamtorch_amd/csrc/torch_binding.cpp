@@ -1,0 +1,324 @@
+// PyTorch-ROCm operator registration for the MAM hot path.  This file is plumbing only: it
+// checks tensors, allocates outputs / workspace through torch's caching allocator, picks up the
+// current HIP stream and calls the C ABI of libmam_hip.so (include/mam_hip.h).  No kernels here.
+//
+// Operator names and schemas are those of SSIGPRO/mamtorch 1.5.2
+// (mamtorch/kernel/v1/csrc/register_functions.cpp:21-24,
+//  mamtorch/kernel/v4/csrc/register_functions.cpp:10-14,
+//  mamtorch/sparse/kernel/v1/csrc/cuda/register_functions.cu:18-28), so the reference's Python
+// wrappers, fake kernels and autograd formulas bind to them unchanged.  Operators without an
+// upstream name (weight-layout variants, selection_count, sparse MAM) are additions.
+//
+// Unlike the reference (whose TORCH_CHECKs are commented out,
+// mamtorch/kernel/v1/csrc/cuda/fullyconnected.cu:181-189) every entry validates dtype, shape,
+// device and contiguity and raises RuntimeError; launches go to the current stream under a
+// device guard instead of the legacy default stream.
+#include <ATen/ATen.h>
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <vector>
+
+#include "../../include/mam_hip.h"
+
+namespace {
+
+void *current_stream(const at::Tensor &t)
+{
+    return static_cast<void *>(c10::hip::getCurrentHIPStream(t.get_device()).stream());
+}
+
+void check_rc(int rc, const char *what)
+{
+    TORCH_CHECK(rc == MAM_OK, what, " failed: ", mam_error_string(rc), " (", mam_last_error(), ")");
+}
+
+void check_f32_2d(const at::Tensor &t, const char *name)
+{
+    TORCH_CHECK(t.is_cuda(), name, " must be on the GPU");
+    TORCH_CHECK(t.scalar_type() == at::kFloat, name, " must be float32");
+    TORCH_CHECK(t.dim() == 2, name, " must be 2-dimensional");
+}
+
+// Rows may be strided (a narrow() along the last dimension), elements within a row may not.
+int64_t row_stride(const at::Tensor &t, const char *name)
+{
+    TORCH_CHECK(t.size(1) <= 1 || t.stride(1) == 1, name, " must have unit stride in its last dimension");
+    if (t.size(0) <= 1) return std::max<int64_t>(t.size(1), 1);
+    TORCH_CHECK(t.stride(0) >= t.size(1), name, " has overlapping rows");
+    return t.stride(0);
+}
+
+void check_same_device(const at::Tensor &a, const at::Tensor &b, const char *name)
+{
+    TORCH_CHECK(a.device() == b.device(), name, " is on a different device");
+}
+
+void check_index(const at::Tensor &t, const at::Tensor &like, const char *name)
+{
+    TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt, name, " must be an int32 GPU tensor");
+    TORCH_CHECK(t.sizes() == like.sizes(), name, " has the wrong shape");
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+    check_same_device(t, like, name);
+}
+
+at::Tensor workspace_for(size_t bytes, const at::Tensor &like)
+{
+    if (bytes == 0) return at::Tensor();
+    return at::empty({static_cast<int64_t>(bytes)}, like.options().dtype(at::kByte));
+}
+
+struct FwdShape { int64_t N, K, M; };
+
+FwdShape check_forward(const at::Tensor &a, const at::Tensor &w, int layout,
+                       const c10::optional<at::Tensor> &bias)
+{
+    check_f32_2d(a, "a");
+    check_f32_2d(w, layout == MAM_W_MK ? "weight" : "b");
+    check_same_device(a, w, "the weight operand");
+    FwdShape s{a.size(0), a.size(1), layout == MAM_W_MK ? w.size(0) : w.size(1)};
+    TORCH_CHECK((layout == MAM_W_MK ? w.size(1) : w.size(0)) == s.K,
+                "inner dimensions do not match: a is (", a.size(0), ",", a.size(1), "), the weight operand is (",
+                w.size(0), ",", w.size(1), ")");
+    TORCH_CHECK(s.K > 0 || s.N == 0 || s.M == 0, "in_features must be positive");
+    if (bias.has_value() && bias->defined()) {
+        TORCH_CHECK(bias->is_cuda() && bias->scalar_type() == at::kFloat && bias->dim() == 1 &&
+                        bias->size(0) == s.M && bias->is_contiguous(),
+                    "bias must be a contiguous float32 GPU vector of out_features elements");
+        check_same_device(a, *bias, "bias");
+    }
+    return s;
+}
+
+const float *bias_ptr(const c10::optional<at::Tensor> &bias)
+{
+    return (bias.has_value() && bias->defined()) ? bias->data_ptr<float>() : nullptr;
+}
+
+std::vector<at::Tensor> forward_impl(const at::Tensor &a, const at::Tensor &w, int layout,
+                                     const c10::optional<at::Tensor> &bias)
+{
+    const FwdShape s = check_forward(a, w, layout, bias);
+    const c10::DeviceGuard guard(a.device());
+    auto c = at::empty({s.N, s.M}, a.options());
+    auto argmax = at::empty({s.N, s.M}, a.options().dtype(at::kInt));
+    auto argmin = at::empty({s.N, s.M}, a.options().dtype(at::kInt));
+    if (s.N == 0 || s.M == 0) return {c, argmax, argmin};
+    const size_t ws_bytes = mam_fc_forward_workspace(s.N, s.K, s.M);
+    auto ws = workspace_for(ws_bytes, a);
+    check_rc(mam_fc_forward(a.data_ptr<float>(), row_stride(a, "a"), w.data_ptr<float>(),
+                            row_stride(w, "the weight operand"), layout, bias_ptr(bias),
+                            c.data_ptr<float>(), argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
+                            s.N, s.K, s.M, ws.defined() ? ws.data_ptr() : nullptr, ws_bytes,
+                            current_stream(a)),
+             "mam_fc_forward");
+    return {c, argmax, argmin};
+}
+
+at::Tensor forward_values_impl(const at::Tensor &a, const at::Tensor &w, int layout,
+                               const c10::optional<at::Tensor> &bias)
+{
+    const FwdShape s = check_forward(a, w, layout, bias);
+    const c10::DeviceGuard guard(a.device());
+    auto c = at::empty({s.N, s.M}, a.options());
+    if (s.N == 0 || s.M == 0) return c;
+    const size_t ws_bytes = mam_fc_forward_values_workspace(s.N, s.K, s.M);
+    auto ws = workspace_for(ws_bytes, a);
+    check_rc(mam_fc_forward_values(a.data_ptr<float>(), row_stride(a, "a"), w.data_ptr<float>(),
+                                   row_stride(w, "the weight operand"), layout, bias_ptr(bias),
+                                   c.data_ptr<float>(), s.N, s.K, s.M,
+                                   ws.defined() ? ws.data_ptr() : nullptr, ws_bytes, current_stream(a)),
+             "mam_fc_forward_values");
+    return c;
+}
+
+std::vector<at::Tensor> backward_impl(const at::Tensor &a, const at::Tensor &w, int layout,
+                                      const at::Tensor &grad, const at::Tensor &argmax,
+                                      const at::Tensor &argmin)
+{
+    const FwdShape s = check_forward(a, w, layout, c10::nullopt);
+    check_f32_2d(grad, "grad");
+    TORCH_CHECK(grad.size(0) == s.N && grad.size(1) == s.M, "grad must be (batch, out_features)");
+    check_same_device(a, grad, "grad");
+    check_index(argmax, grad, "argmax");
+    check_index(argmin, grad, "argmin");
+    const c10::DeviceGuard guard(a.device());
+    const at::Tensor g = grad.contiguous();
+    auto a_grad = at::empty({s.N, s.K}, a.options());
+    auto w_grad = at::empty(w.sizes(), w.options());
+    check_rc(mam_fc_backward(a.data_ptr<float>(), row_stride(a, "a"), w.data_ptr<float>(),
+                             row_stride(w, "the weight operand"), layout, g.data_ptr<float>(),
+                             argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
+                             a_grad.data_ptr<float>(), w_grad.data_ptr<float>(), s.N, s.K, s.M,
+                             current_stream(a)),
+             "mam_fc_backward");
+    return {a_grad, w_grad};
+}
+
+// ---- reference operator names: b is (in_features, out_features).  Rows of a and b may be
+// strided views (the module's splits > 1 path narrows them); the reference reads such views as if
+// they were contiguous. ----
+std::vector<at::Tensor> fullyconnected(at::Tensor a, at::Tensor b)
+{
+    return forward_impl(a, b, MAM_W_KM, c10::nullopt);
+}
+
+at::Tensor fullyconnected_fast(at::Tensor a, at::Tensor b)
+{
+    return forward_values_impl(a, b, MAM_W_KM, c10::nullopt);
+}
+
+std::vector<at::Tensor> fullyconnected_backward(at::Tensor a, at::Tensor b, at::Tensor grad,
+                                                at::Tensor argmax, at::Tensor argmin)
+{
+    return backward_impl(a, b, MAM_W_KM, grad, argmax, argmin);
+}
+
+// ---- additions: weight in the module's own (out_features, in_features) layout, fused bias ----
+std::vector<at::Tensor> fullyconnected_wt(const at::Tensor &a, const at::Tensor &weight,
+                                          const c10::optional<at::Tensor> &bias)
+{
+    return forward_impl(a, weight, MAM_W_MK, bias);
+}
+
+at::Tensor fullyconnected_fast_wt(const at::Tensor &a, const at::Tensor &weight,
+                                  const c10::optional<at::Tensor> &bias)
+{
+    return forward_values_impl(a, weight, MAM_W_MK, bias);
+}
+
+std::vector<at::Tensor> fullyconnected_wt_backward(const at::Tensor &a, const at::Tensor &weight,
+                                                   const at::Tensor &grad, const at::Tensor &argmax,
+                                                   const at::Tensor &argmin)
+{
+    return backward_impl(a, weight, MAM_W_MK, grad, argmax, argmin);
+}
+
+void selection_count(const at::Tensor &argmax, const at::Tensor &argmin, at::Tensor max_count,
+                     at::Tensor min_count, int64_t mode)
+{
+    TORCH_CHECK(argmax.dim() == 2, "argmax must be (batch, out_features)");
+    check_index(argmax, argmax, "argmax");
+    check_index(argmin, argmax, "argmin");
+    TORCH_CHECK(max_count.dim() == 2 && max_count.size(0) == argmax.size(1),
+                "max_count must be (out_features, in_features)");
+    check_index(max_count, max_count, "max_count");
+    check_index(min_count, max_count, "min_count");
+    check_same_device(argmax, max_count, "max_count");
+    const c10::DeviceGuard guard(argmax.device());
+    check_rc(mam_selection_count(argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
+                                 max_count.data_ptr<int32_t>(), min_count.data_ptr<int32_t>(),
+                                 argmax.size(0), argmax.size(1), max_count.size(1), (int)mode,
+                                 current_stream(argmax)),
+             "mam_selection_count");
+}
+
+// ---- CSR-sparse MAM: w_csr is the pruned weight (out_features, in_features) ----
+struct CsrParts { at::Tensor crow, col, val; };
+
+CsrParts csr_parts(const at::Tensor &w_csr, const at::Tensor &a)
+{
+    TORCH_CHECK(w_csr.layout() == at::kSparseCsr, "w_csr must be a torch.sparse_csr tensor");
+    TORCH_CHECK(w_csr.dim() == 2 && w_csr.size(1) == a.size(1), "w_csr must be (out_features, in_features)");
+    CsrParts p{w_csr.crow_indices().to(at::kLong).contiguous(), w_csr.col_indices().to(at::kLong).contiguous(),
+               w_csr.values().contiguous()};
+    TORCH_CHECK(p.val.scalar_type() == at::kFloat, "w_csr values must be float32");
+    TORCH_CHECK(p.val.is_cuda() && p.val.device() == a.device(), "w_csr is on a different device");
+    return p;
+}
+
+std::vector<at::Tensor> sparse_fullyconnected(const at::Tensor &a, const at::Tensor &w_csr)
+{
+    check_f32_2d(a, "a");
+    const CsrParts p = csr_parts(w_csr, a);
+    const int64_t N = a.size(0), K = a.size(1), M = w_csr.size(0);
+    TORCH_CHECK(K > 0 || N == 0 || M == 0, "in_features must be positive");
+    const c10::DeviceGuard guard(a.device());
+    auto c = at::empty({N, M}, a.options());
+    auto argmax = at::empty({N, M}, a.options().dtype(at::kInt));
+    auto argmin = at::empty({N, M}, a.options().dtype(at::kInt));
+    if (N == 0 || M == 0) return {c, argmax, argmin};
+    check_rc(mam_csr_fc_forward(a.data_ptr<float>(), row_stride(a, "a"), p.crow.data_ptr<int64_t>(),
+                                p.col.data_ptr<int64_t>(), p.val.data_ptr<float>(), nullptr,
+                                c.data_ptr<float>(), argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
+                                N, K, M, nullptr, 0, current_stream(a)),
+             "mam_csr_fc_forward");
+    return {c, argmax, argmin};
+}
+
+std::vector<at::Tensor> sparse_fullyconnected_backward(const at::Tensor &a, const at::Tensor &w_csr,
+                                                       const at::Tensor &grad, const at::Tensor &argmax,
+                                                       const at::Tensor &argmin)
+{
+    check_f32_2d(a, "a");
+    check_f32_2d(grad, "grad");
+    const CsrParts p = csr_parts(w_csr, a);
+    const int64_t N = a.size(0), K = a.size(1), M = w_csr.size(0);
+    TORCH_CHECK(grad.size(0) == N && grad.size(1) == M, "grad must be (batch, out_features)");
+    check_index(argmax, grad, "argmax");
+    check_index(argmin, grad, "argmin");
+    const c10::DeviceGuard guard(a.device());
+    const at::Tensor g = grad.contiguous();
+    auto a_grad = at::empty({N, K}, a.options());
+    auto val_grad = at::empty_like(p.val);
+    check_rc(mam_csr_fc_backward(a.data_ptr<float>(), row_stride(a, "a"), p.crow.data_ptr<int64_t>(),
+                                 p.col.data_ptr<int64_t>(), p.val.data_ptr<float>(), g.data_ptr<float>(),
+                                 argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
+                                 a_grad.data_ptr<float>(), val_grad.data_ptr<float>(), N, K, M,
+                                 p.val.numel(), current_stream(a)),
+             "mam_csr_fc_backward");
+    return {a_grad, val_grad};
+}
+
+}  // namespace
+
+TORCH_LIBRARY(mamtorch_kernel_v1, m)
+{
+    m.def("fullyconnected(Tensor a, Tensor b) -> Tensor[]");
+    m.def("fullyconnected_backward(Tensor a, Tensor b, Tensor grad, Tensor argmax, Tensor argmin) -> Tensor[]");
+}
+
+TORCH_LIBRARY(mamtorch_kernel_v4, m)
+{
+    m.def("fullyconnected(Tensor a, Tensor b) -> Tensor[]");
+    m.def("fullyconnected_fast(Tensor a, Tensor b) -> Tensor");
+    m.def("fullyconnected_backward(Tensor a, Tensor b, Tensor grad, Tensor argmax, Tensor argmin) -> Tensor[]");
+    m.def("fullyconnected_wt(Tensor a, Tensor weight, Tensor? bias) -> Tensor[]");
+    m.def("fullyconnected_fast_wt(Tensor a, Tensor weight, Tensor? bias) -> Tensor");
+    m.def("fullyconnected_wt_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin) -> Tensor[]");
+    m.def("selection_count(Tensor argmax, Tensor argmin, Tensor(a!) max_count, Tensor(b!) min_count, int mode) -> ()");
+}
+
+TORCH_LIBRARY(mamtorch_kernel_sparsev1, m)
+{
+    m.def("fullyconnected(Tensor a, Tensor w_csr) -> Tensor[]");
+    m.def("fullyconnected_backward(Tensor a, Tensor w_csr, Tensor grad, Tensor argmax, Tensor argmin) -> Tensor[]");
+}
+
+// On PyTorch-ROCm the HIP device is served by the CUDA dispatch key.
+TORCH_LIBRARY_IMPL(mamtorch_kernel_v1, CUDA, m)
+{
+    m.impl("fullyconnected", &fullyconnected);
+    m.impl("fullyconnected_backward", &fullyconnected_backward);
+}
+
+TORCH_LIBRARY_IMPL(mamtorch_kernel_v4, CUDA, m)
+{
+    m.impl("fullyconnected", &fullyconnected);
+    m.impl("fullyconnected_fast", &fullyconnected_fast);
+    m.impl("fullyconnected_backward", &fullyconnected_backward);
+    m.impl("fullyconnected_wt", &fullyconnected_wt);
+    m.impl("fullyconnected_fast_wt", &fullyconnected_fast_wt);
+    m.impl("fullyconnected_wt_backward", &fullyconnected_wt_backward);
+    m.impl("selection_count", &selection_count);
+}
+
+// The dense operand decides the key for mixed dense / sparse-CSR arguments only when the sparse
+// key is absent, so the sparse operators are registered on the sparse-CSR key, as the reference
+// does for cusparsemm (mamtorch/sparse/kernel/v1/csrc/cuda/register_functions.cu:26-28).
+TORCH_LIBRARY_IMPL(mamtorch_kernel_sparsev1, SparseCsrCUDA, m)
+{
+    m.impl("fullyconnected", &sparse_fullyconnected);
+    m.impl("fullyconnected_backward", &sparse_fullyconnected_backward);
+}

@@ -1,0 +1,127 @@
+"""CPU oracle for the MAM fully-connected hot path -- TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this
+package, and only as the checker.  The shipped package never imports it.
+
+Three independent statements of the same algorithm live here:
+  * ``mam_oracle.c``   -- plain C triple loops (ctypes wrappers below); fast enough for
+                          the medium-size parity cases.
+  * ``torch_port.py``  -- pure-PyTorch, batch-chunked restatement of the reference's
+                          test/reference.py:3-25; it is the CPU baseline timed by bench.py.
+  * ``brute.py``       -- pure-Python loops over numpy float32 scalars for tiny inputs;
+                          it pins the other two.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libmam_oracle.so")
+_lib = None
+
+W_KM = 0  # w is (K, M): the operator's ``b`` operand
+W_MK = 1  # w is (M, K): the module's ``weight`` (out, in)
+
+
+def build(force=False):
+    """Compile mam_oracle.c with gcc (oracle/Makefile)."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.check_call(["make", "-s", "-C", _HERE, "libmam_oracle.so"])
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _f32(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float32))
+
+
+def _i32(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.int32))
+
+
+def _i64(a):
+    return np.ascontiguousarray(np.asarray(a, dtype=np.int64))
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+_I64 = ctypes.c_int64
+
+
+def forward(x, w, layout=W_KM, bias=None):
+    """Returns (c, argmax, argmin) as numpy arrays; x (N,K), w (K,M) or (M,K)."""
+    x, w = _f32(x), _f32(w)
+    N, K = x.shape
+    M = w.shape[1] if layout == W_KM else w.shape[0]
+    assert (w.shape[0] if layout == W_KM else w.shape[1]) == K
+    b = None if bias is None else _f32(bias)
+    c = np.empty((N, M), np.float32)
+    amax = np.empty((N, M), np.int32)
+    amin = np.empty((N, M), np.int32)
+    lib().mam_oracle_forward(_p(x), _I64(K), _p(w), _I64(w.shape[1]), ctypes.c_int(layout), _p(b),
+                             _p(c), _p(amax), _p(amin), _I64(N), _I64(K), _I64(M))
+    return c, amax, amin
+
+
+def backward(x, w, grad, argmax, argmin, layout=W_KM):
+    """Returns (x_grad (N,K), w_grad in the layout of w)."""
+    x, w, grad = _f32(x), _f32(w), _f32(grad)
+    argmax, argmin = _i32(argmax), _i32(argmin)
+    N, K = x.shape
+    M = grad.shape[1]
+    xg = np.empty((N, K), np.float32)
+    wg = np.empty(w.shape, np.float32)
+    lib().mam_oracle_backward(_p(x), _I64(K), _p(w), _I64(w.shape[1]), ctypes.c_int(layout), _p(grad),
+                              _p(argmax), _p(argmin), _p(xg), _p(wg), _I64(N), _I64(K), _I64(M))
+    return xg, wg
+
+
+def selection_count(argmax, argmin, max_count, min_count, mode=0):
+    """Adds to copies of the (M,K) int32 counters and returns them."""
+    argmax, argmin = _i32(argmax), _i32(argmin)
+    mc, nc = _i32(max_count).copy(), _i32(min_count).copy()
+    N, M = argmax.shape
+    K = mc.shape[1]
+    lib().mam_oracle_selection_count(_p(argmax), _p(argmin), _p(mc), _p(nc), _I64(N), _I64(M), _I64(K),
+                                     ctypes.c_int(mode))
+    return mc, nc
+
+
+def csr_forward(x, crow, col, val, K, bias=None):
+    x, val = _f32(x), _f32(val)
+    crow, col = _i64(crow), _i64(col)
+    N = x.shape[0]
+    M = crow.shape[0] - 1
+    b = None if bias is None else _f32(bias)
+    c = np.empty((N, M), np.float32)
+    amax = np.empty((N, M), np.int32)
+    amin = np.empty((N, M), np.int32)
+    lib().mam_oracle_csr_forward(_p(x), _I64(K), _p(crow), _p(col), _p(val), _p(b), _p(c), _p(amax),
+                                 _p(amin), _I64(N), _I64(K), _I64(M))
+    return c, amax, amin
+
+
+def csr_backward(x, crow, col, val, grad, argmax, argmin):
+    x, val, grad = _f32(x), _f32(val), _f32(grad)
+    crow, col = _i64(crow), _i64(col)
+    argmax, argmin = _i32(argmax), _i32(argmin)
+    N, K = x.shape
+    M = crow.shape[0] - 1
+    xg = np.empty((N, K), np.float32)
+    vg = np.empty(val.shape, np.float32)
+    lib().mam_oracle_csr_backward(_p(x), _I64(K), _p(crow), _p(col), _p(val), _p(grad), _p(argmax),
+                                  _p(argmin), _p(xg), _p(vg), _I64(N), _I64(K), _I64(M))
+    return xg, vg
