@@ -1,0 +1,171 @@
+"""GPU parity of the MAM backward through the C ABI.
+
+Bar: |got - want| <= 1e-5 * |want| + 2^-22 * S, where `want` is the oracle's order-independent
+(fp64-accumulated) sum and S is the sum of the absolute values of the fp32 terms that make up
+that cell.  The second term is the rounding floor of ANY fp32 summation order (the reference's
+atomicAdd order is itself unspecified): where a cell's terms cancel, a relative bound on the
+result alone cannot be met by fp32 adds.  For cells with a single term the bar is plain rtol 1e-5."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import config1, random_case
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+RTOL = 1e-5
+FLOOR = 2.0 ** -22
+
+
+def _check(x, w_mk, grad, amax, amin, what, layouts=(0, 1)):
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    xo, wo = oracle.backward(x.numpy(), w_mk.numpy(), grad.numpy(), amax, amin, oracle.W_MK)
+    xs, ws_ = oracle.backward(x.abs().numpy(), w_mk.abs().numpy(), grad.abs().numpy(), amax, amin, oracle.W_MK)
+
+    def close(got, want, abs_sum, msg):
+        err = np.abs(got.astype(np.float64) - want)
+        tol = RTOL * np.abs(want) + FLOOR * abs_sum + 1e-30
+        bad = np.argwhere(err > tol)
+        assert bad.size == 0, "%s: %d cells out of tolerance, first %s got %r want %r (sum|terms| %r)" % (
+            msg, len(bad), bad[0].tolist(), got[tuple(bad[0])], want[tuple(bad[0])], abs_sum[tuple(bad[0])])
+
+    xd, gd = x.to(dev), grad.to(dev)
+    a1, a2 = torch.tensor(amax).to(dev), torch.tensor(amin).to(dev)
+    for layout in layouts:
+        wd = (w_mk if layout == capi.W_MK else w_mk.T).contiguous().to(dev)
+        xg, wg = capi.fc_backward(xd, wd, gd, a1, a2, layout)
+        torch.cuda.synchronize()
+        wg = wg.cpu().numpy() if layout == capi.W_MK else wg.cpu().numpy().T
+        close(xg.cpu().numpy(), xo, xs, "%s x_grad layout %d" % (what, layout))
+        close(wg, wo, ws_, "%s w_grad layout %d" % (what, layout))
+    return xo, wo
+
+
+def test_known_answers():
+    def conv(v):
+        return [conv(e) for e in v] if isinstance(v, list) else float(v)
+    for kat in json.load(open(os.path.join(GOLDEN, "kat.json"))):
+        if "a" not in kat:
+            continue
+        a = torch.tensor(conv(kat["a"]), dtype=torch.float32)
+        b = torch.tensor(conv(kat["b"]), dtype=torch.float32)
+        g = torch.tensor(conv(kat["grad"]), dtype=torch.float32)
+        xo, wo = _check(a, b.T.contiguous(), g, np.asarray(kat["argmax"], np.int32),
+                        np.asarray(kat["argmin"], np.int32), kat["name"])
+        np.testing.assert_array_equal(xo, np.asarray(kat["a_grad"], np.float32))
+        np.testing.assert_array_equal(wo.T, np.asarray(kat["b_grad"], np.float32))
+
+
+def test_golden_brute_fixtures():
+    data = np.load(os.path.join(GOLDEN, "brute_small.npz"))
+    for i in range(5):
+        f = lambda n: data["case%d_%s" % (i, n)]
+        xo, wo = _check(torch.tensor(f("x")), torch.tensor(f("b")).T.contiguous(), torch.tensor(f("grad")),
+                        f("argmax"), f("argmin"), "fixture %d" % i)
+        np.testing.assert_allclose(xo, f("x_grad"), rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(wo.T, f("b_grad"), rtol=1e-6, atol=1e-7)
+
+
+def test_config1():
+    x, w, bias, grad = config1()
+    _, amax, amin = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+    _check(x, w, grad, amax, amin, "config 1")
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 7), (65, 33, 130), (200, 1001, 70), (17, 9, 300), (300, 257, 31)])
+def test_ragged_shapes(shape):
+    N, K, M = shape
+    x, w, grad = random_case(N, K, M, seed=sum(shape))
+    _, amax, amin = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+    _check(x, w, grad, amax, amin, "shape %s" % (shape,))
+
+
+def test_concentrated_and_duplicate_selections():
+    g = torch.Generator().manual_seed(5)
+    N, K, M = 128, 64, 96
+    x, w, grad = random_case(N, K, M, seed=5)
+    # every output selects the same k for max and min: 2*M terms collide on one x_grad cell per row
+    amax = np.full((N, M), 7, np.int32)
+    _check(x, w, grad, amax, amax.copy(), "all on k=7")
+    # random picks, unrelated to the true extremes (as in the reference's backward benchmark,
+    # test/test.py:316-317)
+    amax = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32).numpy()
+    amin = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32).numpy()
+    _check(x, w, grad, amax, amin, "random picks")
+
+
+def test_k_larger_than_one_lds_histogram():
+    N, K, M = 6, 70000, 40
+    x, w, grad = random_case(N, K, M, seed=9)
+    g = torch.Generator().manual_seed(9)
+    amax = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32).numpy()
+    amin = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32).numpy()
+    amax[0, :] = K - 1
+    amin[0, :] = 0
+    _check(x, w, grad, amax, amin, "K=70000")
+
+
+def test_either_output_can_be_skipped_and_strided_inputs():
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    N, K, M, off, sub = 40, 64, 50, 3, 29
+    x, w, grad = random_case(N, K, M, seed=3)
+    xs, ws = x[:, off:off + sub].contiguous(), w[:, off:off + sub].contiguous()
+    _, amax, amin = oracle.forward(xs.numpy(), ws.numpy(), oracle.W_MK)
+    xo, wo = oracle.backward(xs.numpy(), ws.numpy(), grad.numpy(), amax, amin, oracle.W_MK)
+    xd, wd = x.to(dev).narrow(1, off, sub), w.to(dev).narrow(1, off, sub)
+    a1, a2 = torch.tensor(amax).to(dev), torch.tensor(amin).to(dev)
+    xg, wg = capi.fc_backward(xd, wd, grad.to(dev), a1, a2, capi.W_MK)
+    np.testing.assert_allclose(xg.cpu().numpy(), xo, rtol=RTOL, atol=1e-6)
+    np.testing.assert_allclose(wg.cpu().numpy(), wo, rtol=RTOL, atol=1e-6)
+    xg, none = capi.fc_backward(xd, wd, grad.to(dev), a1, a2, capi.W_MK, want_w=False)
+    assert none is None
+    np.testing.assert_allclose(xg.cpu().numpy(), xo, rtol=RTOL, atol=1e-6)
+    none, wg = capi.fc_backward(xd, wd, grad.to(dev), a1, a2, capi.W_MK, want_x=False)
+    assert none is None
+    np.testing.assert_allclose(wg.cpu().numpy(), wo, rtol=RTOL, atol=1e-6)
+
+
+def test_headline_config2_full_size():
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    N, K, M = 256, 4096, 4096
+    x = torch.randn(N, K, generator=g)
+    w = (torch.rand(M, K, generator=g) * 2 - 1) / 64
+    grad = torch.randn(N, M, generator=g)
+    _, amax, amin = capi.fc_forward(x.to(dev), w.to(dev), capi.W_MK)
+    xo, wo = _check(x, w, grad, amax.cpu().numpy(), amin.cpu().numpy(), "config 2")
+    # at most 2*N*M cells of the weight gradient are touched
+    assert np.count_nonzero(wo) <= 2 * N * M
+    # linearity in grad
+    xd, wd = x.to(dev), w.to(dev)
+    g2 = torch.randn(N, M, generator=g)
+    xa, wa = capi.fc_backward(xd, wd, grad.to(dev), amax, amin, capi.W_MK)
+    xb, wb = capi.fc_backward(xd, wd, g2.to(dev), amax, amin, capi.W_MK)
+    xc, wc = capi.fc_backward(xd, wd, (grad + g2).to(dev), amax, amin, capi.W_MK)
+    assert torch.allclose(xa + xb, xc, rtol=1e-4, atol=1e-5)
+    assert torch.allclose(wa + wb, wc, rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dims", [(768, 3072), (3072, 768)])
+def test_vit_mlp_config3_shapes(dims):
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    K, M = dims
+    N = 12608
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(N, K, generator=g)
+    w = (torch.rand(M, K, generator=g) * 2 - 1) / K ** 0.5
+    grad = torch.randn(N, M, generator=g)
+    _, amax, amin = capi.fc_forward(x.to(dev), w.to(dev), capi.W_MK)
+    _check(x, w, grad, amax.cpu().numpy(), amin.cpu().numpy(), "config 3", layouts=(1,))

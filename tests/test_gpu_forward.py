@@ -1,0 +1,269 @@
+"""GPU parity of the dense MAM forward, driven through the C ABI (mamtorch_amd.capi).
+Bar: values bit-exact (fp32 bit patterns), argmax/argmin exactly equal, against the CPU oracle."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import assert_bits_equal, assert_index_equal, config1, random_case
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _dev():
+    return torch.device("cuda:0")
+
+
+def _run_both_layouts(x, w_mk, bias=None, what=""):
+    """x (N,K), w_mk (M,K) CPU tensors.  Checks forward (+values-only) in both layouts vs the oracle."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    want = oracle.forward(x.numpy(), w_mk.numpy(), oracle.W_MK, None if bias is None else bias.numpy())
+    xd = x.to(dev)
+    bd = None if bias is None else bias.to(dev)
+    for layout, w in ((capi.W_MK, w_mk.contiguous()), (capi.W_KM, w_mk.T.contiguous())):
+        wd = w.to(dev)
+        c, amax, amin = capi.fc_forward(xd, wd, layout, bd)
+        cv = capi.fc_forward_values(xd, wd, layout, bd)
+        torch.cuda.synchronize()
+        tag = "%s layout=%d" % (what, layout)
+        assert_bits_equal(c.cpu().numpy(), want[0], tag + " c")
+        assert_index_equal(amax.cpu().numpy(), want[1], tag + " argmax")
+        assert_index_equal(amin.cpu().numpy(), want[2], tag + " argmin")
+        assert_bits_equal(cv.cpu().numpy(), want[0], tag + " values-only c")
+    return want
+
+
+def test_known_answers():
+    def conv(v):
+        return [conv(e) for e in v] if isinstance(v, list) else float(v)
+    for kat in json.load(open(os.path.join(GOLDEN, "kat.json"))):
+        if "a" not in kat:
+            continue
+        a = torch.tensor(conv(kat["a"]), dtype=torch.float32)
+        b = torch.tensor(conv(kat["b"]), dtype=torch.float32)
+        c, amax, amin = _run_both_layouts(a, b.T.contiguous(), what=kat["name"])
+        assert_bits_equal(c, np.asarray(conv(kat["c"]), np.float32), kat["name"])
+        assert amax.tolist() == kat["argmax"] and amin.tolist() == kat["argmin"]
+
+
+def test_golden_brute_fixtures():
+    data = np.load(os.path.join(GOLDEN, "brute_small.npz"))
+    for i in range(5):
+        f = lambda n: torch.tensor(data["case%d_%s" % (i, n)])
+        c, amax, amin = _run_both_layouts(f("x"), f("b").T.contiguous(), f("bias"), "fixture %d" % i)
+        assert_bits_equal(c, data["case%d_c" % i], "fixture %d c" % i)
+        assert_index_equal(amax, data["case%d_argmax" % i], "fixture %d argmax" % i)
+        assert_index_equal(amin, data["case%d_argmin" % i], "fixture %d argmin" % i)
+
+
+def test_config1_bit_exact():
+    x, w, bias, _ = config1()
+    _run_both_layouts(x, w, bias, "config 1")
+    _run_both_layouts(x, w, None, "config 1 no bias")
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (1, 7, 1), (2, 3, 5), (63, 31, 127), (64, 32, 128), (65, 33, 129),
+                                   (130, 257, 70), (17, 1001, 19), (300, 8, 300), (5, 4097, 9)])
+def test_ragged_shapes(shape):
+    N, K, M = shape
+    x, w, _ = random_case(N, K, M, seed=N + K + M)
+    _run_both_layouts(x, w, None, "shape %s" % (shape,))
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_shapes_like_the_reference_test(seed):
+    # the reference draws n, m, l uniformly from [10, 1000] (test/test.py:12-14)
+    rng = np.random.default_rng(100 + seed)
+    N, K, M = (int(v) for v in rng.integers(10, 1001, 3))
+    x, w, _ = random_case(N, K, M, seed)
+    _run_both_layouts(x, w, None, "random %d,%d,%d" % (N, K, M))
+
+
+def test_ties_take_the_lowest_index():
+    g = torch.Generator().manual_seed(1)
+    N, K, M = 70, 200, 140
+    # coarse values: products collide constantly, including exact zeros and +-0
+    x = torch.round(torch.randn(N, K, generator=g) * 2)
+    w = torch.round(torch.randn(M, K, generator=g) * 2)
+    want = _run_both_layouts(x, w, None, "quantised")
+    prod = x.numpy()[:, :, None] * w.numpy().T[None, :, :]
+    tied = (prod == prod.max(axis=1, keepdims=True)).sum(axis=1) > 1
+    assert tied.mean() > 0.5                     # the case really is dominated by tied maxima
+    # all products equal
+    _run_both_layouts(torch.ones(9, 50), torch.full((11, 50), 5.0), None, "all equal")
+    # a zero row of x: every product is +-0, the sign comes from the first product
+    x = torch.randn(6, 40, generator=g); x[2] = 0.0; x[4] = -0.0
+    w = torch.randn(9, 40, generator=g)
+    _run_both_layouts(x, w, None, "zero rows")
+    # duplicate columns of k far apart (different LDS tiles, different groups of 8)
+    x = torch.randn(20, 300, generator=g); w = torch.randn(33, 300, generator=g)
+    x[:, 290] = x[:, 3]; w[:, 290] = w[:, 3]; x[:, 3] *= 50; x[:, 290] *= 50
+    want = _run_both_layouts(x, w, None, "far duplicates")
+    assert not (want[1] == 290).any() and not (want[2] == 290).any()
+
+
+def test_extremes_that_the_reference_kernel_gets_wrong():
+    g = torch.Generator().manual_seed(2)
+    # all products negative (the reference's max accumulator starts at +1.18e-38)
+    x = torch.rand(10, 64, generator=g) + 0.5
+    w = -(torch.rand(12, 64, generator=g) + 0.5)
+    want = _run_both_layouts(x, w, None, "all negative")
+    assert (want[0] < 0).all()
+    # subnormal products must not be flushed
+    x = torch.full((4, 16), 1e-20) * (torch.rand(4, 16, generator=g) + 0.5)
+    w = torch.full((5, 16), 1e-20) * (torch.rand(5, 16, generator=g) - 0.5)
+    want = _run_both_layouts(x, w, None, "subnormal")
+    assert np.abs(want[0]).max() < 1.2e-38 and np.abs(want[0]).max() > 0
+    # huge dynamic range and infinities of the same sign
+    x = torch.randn(8, 40, generator=g) * 1e30
+    w = torch.randn(7, 40, generator=g) * 1e30
+    want = _run_both_layouts(x, w, None, "overflow to inf")
+    assert np.isinf(want[0]).any() or np.isnan(want[0]).any()
+
+
+def test_pruned_dense_weight_with_many_zeros():
+    g = torch.Generator().manual_seed(3)
+    N, K, M = 96, 512, 160
+    x = torch.randn(N, K, generator=g)
+    w = torch.randn(M, K, generator=g) * (torch.rand(M, K, generator=g) < 0.05)
+    w[0] = 0.0
+    w[1] = -w[1].abs()
+    _run_both_layouts(x, w, None, "95% zeros")
+
+
+def test_strided_rows_and_unaligned_views():
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(4)
+    N, K, M, off, sub = 50, 96, 70, 5, 37
+    x = torch.randn(N, K, generator=g); w = torch.randn(M, K, generator=g)
+    xd, wd = x.to(dev), w.to(dev)
+    # narrow along K: row stride stays K, base pointer is only 4-byte aligned
+    xv, wv = xd.narrow(1, off, sub), wd.narrow(1, off, sub)
+    c, amax, amin = capi.fc_forward(xv, wv, capi.W_MK)
+    want = oracle.forward(x[:, off:off + sub].numpy(), w[:, off:off + sub].numpy(), oracle.W_MK)
+    torch.cuda.synchronize()
+    assert_bits_equal(c.cpu().numpy(), want[0], "narrow c")
+    assert_index_equal(amax.cpu().numpy(), want[1], "narrow argmax")
+    assert_index_equal(amin.cpu().numpy(), want[2], "narrow argmin")
+    # (K, M) operand narrowed along K (rows) and along M (row stride > M)
+    b = w.T.contiguous().to(dev)
+    c, amax, amin = capi.fc_forward(xv, b.narrow(0, off, sub), capi.W_KM)
+    torch.cuda.synchronize()
+    assert_bits_equal(c.cpu().numpy(), want[0], "narrow KM c")
+    bm = b.narrow(1, 3, 41)
+    c, amax, amin = capi.fc_forward(xd, bm, capi.W_KM)
+    want = oracle.forward(x.numpy(), w[3:44].numpy(), oracle.W_MK)
+    torch.cuda.synchronize()
+    assert_bits_equal(c.cpu().numpy(), want[0], "column-narrowed KM c")
+    assert_index_equal(amax.cpu().numpy(), want[1], "column-narrowed KM argmax")
+
+
+@pytest.mark.parametrize("shape", [(256, 4096, 512), (64, 8192, 128), (100, 1000, 257), (256, 2048, 1024)])
+def test_split_k_path(shape):
+    from mamtorch_amd import capi
+
+    N, K, M = shape
+    assert capi.lib().mam_fc_forward_workspace(N, K, M) > 0, "shape no longer exercises split-K"
+    x, w, _ = random_case(N, K, M, seed=7, w_scale=1.0 / K ** 0.5)
+    bias = torch.randn(M, generator=torch.Generator().manual_seed(8))
+    _run_both_layouts(x, w, bias, "split-K %s" % (shape,))
+    # ties across splits: one dominant column of k planted again in every K range
+    x2, w2 = x.clone(), w.clone()
+    x2[:, 5] *= 100
+    planted = list(range(100, K, K // 8))
+    for k in planted:
+        x2[:, k] = x2[:, 5]
+        w2[:, k] = w2[:, 5]
+    want = _run_both_layouts(x2, w2, None, "split-K ties %s" % (shape,))
+    assert (want[1] == 5).mean() > 0.3 and (want[2] == 5).mean() > 0.3
+    assert not np.isin(want[1], planted).any() and not np.isin(want[2], planted).any()
+
+
+def test_workspace_is_required_and_checked():
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    N, K, M = 256, 4096, 512
+    x, w, _ = random_case(N, K, M, seed=1)
+    need = capi.lib().mam_fc_forward_workspace(N, K, M)
+    small = torch.empty(need // 2, dtype=torch.uint8, device=dev)
+    with pytest.raises(capi.MamError) as e:
+        capi.fc_forward(x.to(dev), w.to(dev), capi.W_MK, workspace=small)
+    assert e.value.code == -3 and "workspace" in str(e.value)
+
+
+def test_headline_config2_full_size():
+    """N256 K4096 M4096, x~N(0,1), W~U(+-1/64): every value and index against the C oracle."""
+    g = torch.Generator().manual_seed(0)
+    N, K, M = 256, 4096, 4096
+    x = torch.randn(N, K, generator=g)
+    w = (torch.rand(M, K, generator=g) * 2 - 1) / 64
+    _run_both_layouts(x, w, None, "config 2")
+
+
+@pytest.mark.parametrize("dims", [(768, 3072), (3072, 768)])
+def test_vit_mlp_config3_shapes(dims):
+    """N = 64 x 197 = 12608 token rows; oracle on a fixed sample of rows, size-independent
+    properties on all rows."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    K, M = dims
+    N = 12608
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(N, K, generator=g)
+    w = (torch.rand(M, K, generator=g) * 2 - 1) / K ** 0.5
+    xd, wd = x.to(dev), w.to(dev)
+    c, amax, amin = capi.fc_forward(xd, wd, capi.W_MK)
+    cv = capi.fc_forward_values(xd, wd, capi.W_MK)
+    torch.cuda.synchronize()
+    rows = torch.arange(0, N, 13)
+    want = oracle.forward(x[rows].numpy(), w.numpy(), oracle.W_MK)
+    assert_bits_equal(c[rows.to(dev)].cpu().numpy(), want[0], "config 3 c")
+    assert_index_equal(amax[rows.to(dev)].cpu().numpy(), want[1], "config 3 argmax")
+    assert_index_equal(amin[rows.to(dev)].cpu().numpy(), want[2], "config 3 argmin")
+    assert torch.equal(c, cv)
+    # the selected products reproduce c on every row
+    pm = torch.gather(xd, 1, amax.long()) * wd[torch.arange(M, device=dev)[None, :], amax.long()]
+    pn = torch.gather(xd, 1, amin.long()) * wd[torch.arange(M, device=dev)[None, :], amin.long()]
+    assert torch.equal(pm + pn, c)
+    # permuting the batch rows permutes the outputs
+    perm = torch.randperm(N, generator=g).to(dev)
+    c2, amax2, amin2 = capi.fc_forward(xd[perm].contiguous(), wd, capi.W_MK)
+    assert torch.equal(c2, c[perm]) and torch.equal(amax2, amax[perm]) and torch.equal(amin2, amin[perm])
+
+
+@pytest.mark.parametrize("M", [1024, 4096])
+def test_large_batch_inference_config4(M):
+    """N16384 K4096, x~U(-1,1), W~N(0,0.02): oracle on sampled rows + properties on all."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    N, K = 16384, 4096
+    g = torch.Generator().manual_seed(M)
+    x = torch.rand(N, K, generator=g) * 2 - 1
+    w = torch.randn(M, K, generator=g) * 0.02
+    xd, wd = x.to(dev), w.to(dev)
+    c, amax, amin = capi.fc_forward(xd, wd, capi.W_MK)
+    torch.cuda.synchronize()
+    rows = torch.arange(5, N, 257)
+    want = oracle.forward(x[rows].numpy(), w.numpy(), oracle.W_MK)
+    assert_bits_equal(c[rows.to(dev)].cpu().numpy(), want[0], "config 4 c")
+    assert_index_equal(amax[rows.to(dev)].cpu().numpy(), want[1], "config 4 argmax")
+    assert_index_equal(amin[rows.to(dev)].cpu().numpy(), want[2], "config 4 argmin")
+    cols = torch.arange(M, device=dev)[None, :]
+    pm = torch.gather(xd, 1, amax.long()) * wd[cols, amax.long()]
+    pn = torch.gather(xd, 1, amin.long()) * wd[cols, amin.long()]
+    assert torch.equal(pm + pn, c)
+    assert bool((pm >= pn).all())
+    # the (K, M) operand gives the same answer
+    c2, amax2, amin2 = capi.fc_forward(xd[:2048], wd.T.contiguous(), capi.W_KM)
+    assert torch.equal(c2, c[:2048]) and torch.equal(amax2, amax[:2048]) and torch.equal(amin2, amin[:2048])

@@ -1,0 +1,244 @@
+"""Pins the CPU oracle (oracle/mam_oracle.c, oracle/torch_port.py) without the reference:
+hand-derived known answers, an independent pure-Python brute force, closed-form special cases,
+autograd of a gather formulation and fp64 finite differences.  CPU only."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import brute, torch_port
+from helpers import assert_bits_equal, assert_index_equal, config1, pruned_csr
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _arr(v, dtype=np.float32):
+    def conv(e):
+        if isinstance(e, list):
+            return [conv(i) for i in e]
+        return float(e) if isinstance(e, str) else e
+    return np.asarray(conv(v), dtype=dtype)
+
+
+def _kats():
+    with open(os.path.join(GOLDEN, "kat.json")) as f:
+        return json.load(f)
+
+
+@pytest.mark.parametrize("kat", [k for k in _kats() if "a" in k], ids=lambda k: k["name"])
+def test_known_answers_forward_backward(kat):
+    a, b, g = _arr(kat["a"]), _arr(kat["b"]), _arr(kat["grad"])
+    for fwd in (lambda: oracle.forward(a, b),
+                lambda: oracle.forward(a, np.ascontiguousarray(b.T), oracle.W_MK),
+                lambda: brute.forward(a, b),
+                lambda: tuple(t.numpy() for t in torch_port.forward(torch.tensor(a), torch.tensor(b)))):
+        c, amax, amin = fwd()
+        assert_bits_equal(c, _arr(kat["c"]), kat["name"] + " c")
+        assert_index_equal(amax, _arr(kat["argmax"], np.int32), kat["name"] + " argmax")
+        assert_index_equal(amin, _arr(kat["argmin"], np.int32), kat["name"] + " argmin")
+    amax, amin = _arr(kat["argmax"], np.int32), _arr(kat["argmin"], np.int32)
+    xg, bg = oracle.backward(a, b, g, amax, amin)
+    np.testing.assert_array_equal(xg, _arr(kat["a_grad"]))
+    np.testing.assert_array_equal(bg, _arr(kat["b_grad"]))
+    xg, wg = oracle.backward(a, np.ascontiguousarray(b.T), g, amax, amin, oracle.W_MK)
+    np.testing.assert_array_equal(xg, _arr(kat["a_grad"]))
+    np.testing.assert_array_equal(wg, _arr(kat["b_grad"]).T)
+    xt, bt = torch_port.backward(torch.tensor(a), torch.tensor(b), torch.tensor(g), torch.tensor(amax),
+                                 torch.tensor(amin))
+    np.testing.assert_array_equal(xt.numpy(), _arr(kat["a_grad"]))
+    np.testing.assert_array_equal(bt.numpy(), _arr(kat["b_grad"]))
+
+
+def test_known_answer_selection_count():
+    kat = [k for k in _kats() if k["name"] == "selection_count"][0]
+    amax, amin = _arr(kat["sel_argmax"], np.int32), _arr(kat["sel_argmin"], np.int32)
+    zeros = np.zeros((kat["M"], kat["K"]), np.int32)
+    for impl in (oracle, brute):
+        mc, nc = impl.selection_count(amax, amin, zeros, zeros, mode=0)
+        np.testing.assert_array_equal(mc, _arr(kat["ref_max_count"], np.int32))
+        np.testing.assert_array_equal(nc, zeros)
+        mc, nc = impl.selection_count(amax, amin, zeros, zeros, mode=1)
+        np.testing.assert_array_equal(mc, _arr(kat["hits_max_count"], np.int32))
+        np.testing.assert_array_equal(nc, _arr(kat["hits_min_count"], np.int32))
+    # the literal advanced-index "+= 1" of the module (duplicates do not accumulate)
+    lit = torch_port.selection_count_reference(torch.tensor(amax), torch.tensor(amin),
+                                               torch.zeros((kat["M"], kat["K"]), dtype=torch.int32))
+    np.testing.assert_array_equal(lit.numpy(), _arr(kat["ref_max_count"], np.int32))
+    # the survey's example: three hits on one cell add 1
+    z = torch.zeros(3, 4, dtype=torch.int32)
+    z[torch.tensor([0, 0, 0, 1]), torch.tensor([2, 2, 2, 3])] += 1
+    assert z.tolist() == [[0, 0, 1, 0], [0, 0, 0, 1], [0, 0, 0, 0]]
+
+
+def test_golden_brute_fixtures():
+    data = np.load(os.path.join(GOLDEN, "brute_small.npz"))
+    n_cases = len({k.split("_")[0] for k in data.files})
+    assert n_cases == 5
+    for i in range(n_cases):
+        f = lambda name: data["case%d_%s" % (i, name)]
+        c, amax, amin = oracle.forward(f("x"), f("b"), oracle.W_KM, f("bias"))
+        assert_bits_equal(c, f("c"), "case%d c" % i)
+        assert_index_equal(amax, f("argmax"), "case%d argmax" % i)
+        assert_index_equal(amin, f("argmin"), "case%d argmin" % i)
+        ct, tmax, tmin = torch_port.forward(torch.tensor(f("x")), torch.tensor(f("b")), torch.tensor(f("bias")))
+        assert_bits_equal(ct.numpy(), f("c"), "case%d torch c" % i)
+        assert_index_equal(tmax.numpy(), f("argmax"), "case%d torch argmax" % i)
+        assert_index_equal(tmin.numpy(), f("argmin"), "case%d torch argmin" % i)
+        xg, bg = oracle.backward(f("x"), f("b"), f("grad"), f("argmax"), f("argmin"))
+        np.testing.assert_allclose(xg, f("x_grad"), rtol=1e-6, atol=1e-7)
+        np.testing.assert_allclose(bg, f("b_grad"), rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_three_statements_agree_on_random_inputs(seed):
+    rng = np.random.default_rng(seed)
+    N, K, M = rng.integers(1, 7), rng.integers(1, 24), rng.integers(1, 9)
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    b = rng.standard_normal((K, M)).astype(np.float32)
+    if seed % 2:   # coarse values: many ties and zeros
+        x, b = np.round(x), np.round(b)
+    bias = rng.standard_normal(M).astype(np.float32)
+    cb, b1, b2 = brute.forward(x, b, bias)
+    for c, a1, a2 in (oracle.forward(x, b, oracle.W_KM, bias),
+                      oracle.forward(x, np.ascontiguousarray(b.T), oracle.W_MK, bias),
+                      tuple(t.numpy() for t in torch_port.forward(torch.tensor(x), torch.tensor(b), torch.tensor(bias)))):
+        assert_bits_equal(c, cb, "c")
+        assert_index_equal(a1, b1, "argmax")
+        assert_index_equal(a2, b2, "argmin")
+    g = rng.standard_normal((N, M)).astype(np.float32)
+    xb, bb = brute.backward(x, b, g, b1, b2)
+    xo, bo = oracle.backward(x, b, g, b1, b2)
+    np.testing.assert_allclose(xo, xb, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(bo, bb, rtol=1e-6, atol=1e-7)
+    zeros = np.zeros((M, K), np.int32)
+    for mode in (0, 1):
+        for got, want in zip(oracle.selection_count(b1, b2, zeros + 3, zeros + 1, mode),
+                             brute.selection_count(b1, b2, zeros + 3, zeros + 1, mode)):
+            np.testing.assert_array_equal(got, want)
+
+
+def test_closed_forms():
+    rng = np.random.default_rng(7)
+    # K = 1: C = 2*a*b, both indices 0
+    a = rng.standard_normal((5, 1)).astype(np.float32)
+    b = rng.standard_normal((1, 4)).astype(np.float32)
+    c, amax, amin = oracle.forward(a, b)
+    assert_bits_equal(c, (a * b) + (a * b), "K=1")
+    assert not amax.any() and not amin.any()
+    # non-negative operands: max / min are the largest / smallest product
+    a = np.abs(rng.standard_normal((4, 9))).astype(np.float32)
+    b = np.abs(rng.standard_normal((9, 3))).astype(np.float32)
+    c, amax, amin = oracle.forward(a, b)
+    prod = a[:, :, None] * b[None, :, :]
+    assert_bits_equal(c, prod.max(1) + prod.min(1), "non-negative")
+    np.testing.assert_array_equal(amax, prod.argmax(1))
+    np.testing.assert_array_equal(amin, prod.argmin(1))
+    # one-hot columns of b with a > 0: the max sits at the hot row, the min at the first zero row
+    K, M = 6, 6
+    b = np.eye(K, M, dtype=np.float32)
+    a = (np.abs(rng.standard_normal((3, K))) + 1).astype(np.float32)
+    c, amax, amin = oracle.forward(a, b)
+    np.testing.assert_array_equal(amax, np.tile(np.arange(M), (3, 1)))
+    np.testing.assert_array_equal(amin, np.tile(np.array([1] + [0] * (M - 1)), (3, 1)))
+    assert_bits_equal(c, a[:, :M], "one-hot")
+    # scaling (a*s, b/s) by a power of two leaves everything unchanged
+    a = rng.standard_normal((4, 11)).astype(np.float32)
+    b = rng.standard_normal((11, 5)).astype(np.float32)
+    r0 = oracle.forward(a, b)
+    r1 = oracle.forward(a * np.float32(8), b / np.float32(8))
+    assert_bits_equal(r1[0], r0[0], "scaling")
+    np.testing.assert_array_equal(r1[1], r0[1])
+    np.testing.assert_array_equal(r1[2], r0[2])
+    # permuting k permutes the indices (no ties in continuous data)
+    perm = rng.permutation(11)
+    r2 = oracle.forward(a[:, perm], b[perm, :])
+    assert_bits_equal(r2[0], r0[0], "permutation")
+    np.testing.assert_array_equal(perm[r2[1]], r0[1])
+    np.testing.assert_array_equal(perm[r2[2]], r0[2])
+
+
+def test_backward_matches_autograd_of_gather_formulation():
+    torch.manual_seed(3)
+    N, K, M = 6, 13, 5
+    a = torch.randn(N, K, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(K, M, dtype=torch.float64, requires_grad=True)
+    g = torch.randn(N, M, dtype=torch.float64)
+    prod = a[:, :, None] * b[None, :, :]
+    y = prod.max(dim=1).values + prod.min(dim=1).values
+    y.backward(g)
+    a32, b32, g32 = a.detach().float().numpy(), b.detach().float().numpy(), g.float().numpy()
+    _, amax, amin = oracle.forward(a32, b32)
+    xg, bg = oracle.backward(a32, b32, g32, amax, amin)
+    np.testing.assert_allclose(xg, a.grad.numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(bg, b.grad.numpy(), rtol=1e-5, atol=1e-6)
+    # invariants: both gradients sum to sum g*(selected operand)
+    sel_w = b32[amax, np.arange(M)[None, :]] + b32[amin, np.arange(M)[None, :]]
+    np.testing.assert_allclose(xg.sum(), (g32 * sel_w).sum(), rtol=1e-5)
+    sel_x = np.take_along_axis(a32, amax, 1) + np.take_along_axis(a32, amin, 1)
+    np.testing.assert_allclose(bg.sum(), (g32 * sel_x).sum(), rtol=1e-5)
+
+
+def test_backward_finite_differences_fp64():
+    rng = np.random.default_rng(11)
+    N, K, M = 3, 7, 4
+    a = rng.standard_normal((N, K))
+    b = rng.standard_normal((K, M))
+    g = rng.standard_normal((N, M))
+
+    def loss(a_, b_):
+        p = a_[:, :, None] * b_[None, :, :]
+        return ((p.max(1) + p.min(1)) * g).sum()
+
+    _, amax, amin = oracle.forward(a.astype(np.float32), b.astype(np.float32))
+    xg, bg = oracle.backward(a.astype(np.float32), b.astype(np.float32), g.astype(np.float32), amax, amin)
+    eps = 1e-6
+    for (i, j) in [(0, 0), (1, 3), (2, 6)]:
+        d = np.zeros_like(a); d[i, j] = eps
+        fd = (loss(a + d, b) - loss(a - d, b)) / (2 * eps)
+        assert abs(fd - xg[i, j]) < 1e-4 * max(1.0, abs(fd))
+    for (i, j) in [(0, 0), (4, 2), (6, 3)]:
+        d = np.zeros_like(b); d[i, j] = eps
+        fd = (loss(a, b + d) - loss(a, b - d)) / (2 * eps)
+        assert abs(fd - bg[i, j]) < 1e-4 * max(1.0, abs(fd))
+
+
+def test_config1_c_oracle_vs_torch_port():
+    x, w, bias, grad = config1()
+    c, amax, amin = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK, bias.numpy())
+    ct, tmax, tmin = torch_port.forward(x, w.T.contiguous(), bias)
+    assert_bits_equal(c, ct.numpy(), "config 1 c")
+    assert_index_equal(amax, tmax.numpy(), "config 1 argmax")
+    assert_index_equal(amin, tmin.numpy(), "config 1 argmin")
+    xg, wg = oracle.backward(x.numpy(), w.numpy(), grad.numpy(), amax, amin, oracle.W_MK)
+    xt, bt = torch_port.backward(x, w.T.contiguous(), grad, tmax, tmin)
+    np.testing.assert_allclose(xg, xt.numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(wg, bt.numpy().T, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("density", [0.0, 0.1, 0.5, 1.0])
+def test_csr_oracle_equals_dense_on_densified_weight(density):
+    M, K, N = 12, 20, 5
+    dense, crow, col, val = pruned_csr(M, K, density, seed=5, scale=1.0)
+    if 0 < density < 1:
+        val = val.clone(); val[: int(crow[1])] = -val[: int(crow[1])].abs()   # a row of negative weights
+        dense = torch.zeros(M, K)
+        for m in range(M):
+            dense[m, col[crow[m]:crow[m + 1]]] = val[crow[m]:crow[m + 1]]
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(N, K, generator=g).abs()          # positive inputs: negative rows lose to the zeros
+    x[0] = -x[0]
+    c, amax, amin = oracle.csr_forward(x.numpy(), crow.numpy(), col.numpy(), val.numpy(), K)
+    cd, dmax, dmin = oracle.forward(x.numpy(), dense.numpy(), oracle.W_MK)
+    cb, bmax, bmin = brute.forward(x.numpy(), dense.numpy().T)
+    assert_bits_equal(c, cd, "csr c"); assert_bits_equal(c, cb, "csr c brute")
+    assert_index_equal(amax, dmax, "csr argmax"); assert_index_equal(amax, bmax, "csr argmax brute")
+    assert_index_equal(amin, dmin, "csr argmin"); assert_index_equal(amin, bmin, "csr argmin brute")
+    grad = torch.randn(N, M, generator=g)
+    xg, vg = oracle.csr_backward(x.numpy(), crow.numpy(), col.numpy(), val.numpy(), grad.numpy(), amax, amin)
+    xd, wd = oracle.backward(x.numpy(), dense.numpy(), grad.numpy(), amax, amin, oracle.W_MK)
+    np.testing.assert_allclose(xg, xd, rtol=1e-6, atol=1e-7)
+    rows = np.repeat(np.arange(M), np.diff(crow.numpy()))
+    np.testing.assert_allclose(vg, wd[rows, col.numpy()], rtol=1e-6, atol=1e-7)
