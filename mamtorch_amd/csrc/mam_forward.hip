@@ -9,11 +9,13 @@
 //
 //   * One v_mul_f32 per product; v_max3_f32 / v_min3_f32 fold TWO products into the
 //     running extreme per issue slot.  That is 2 slots per (multiply, max, min) triple.
-//   * Indices are NOT tracked per product.  Products are consumed in groups of G = 8
+//   * Indices are NOT tracked per product.  Products are consumed in groups of G = 16
 //     consecutive k; after a group, one compare + one select per extreme records the group
-//     id if the running extreme strictly improved (0.5 slot per triple).  Because the test is
+//     id if the running extreme strictly improved (0.25 slot per triple).  Because the test is
 //     strict, the recorded group is the one holding the FIRST occurrence of the final extreme.
-//   * An epilogue re-reads the 8 operands of the recorded group, finds the first k whose
+//     Both group ids share one register (16 bits each, written with sub-dword selects), which
+//     is what lets a thread keep 32 outputs and 16 k of X operands in registers at once.
+//   * An epilogue re-reads the 16 operands of the recorded group, finds the first k whose
 //     product equals the extreme, and recomputes the value from that k.  Recomputing also
 //     removes the +0/-0 ambiguity of the hardware max/min, so values and indices are exactly
 //     those of a scalar scan in ascending k with strict comparisons.
@@ -22,7 +24,7 @@
 // W tiles of 32 consecutive k are staged in LDS as [row][k] (row stride 36 floats: 16-byte
 // aligned and conflict-free for ds_read_b128 along k).  A thread owns 4 x 8 outputs, strided
 // by 16 in both directions, so that a wave's W reads cover all banks and its X reads
-// broadcast.  128 of its registers hold (max, min, group-of-max, group-of-min); two
+// broadcast.  96 of its registers hold (max, min, packed group ids); two
 // workgroups share a CU, so each SIMD always has a second wave to issue from while the other
 // waits on LDS or on the tile barrier.  Ragged edges are handled by replicating the last row /
 // column / k on load: a replicated k duplicates an earlier product and can never win a
@@ -40,7 +42,7 @@ constexpr int BN = 64;        // batch rows per workgroup
 constexpr int BM = 128;       // output neurons per workgroup
 constexpr int KT = 32;        // k extent of one LDS tile
 constexpr int LDK = KT + 4;   // LDS row stride in floats
-constexpr int G = 8;          // products per index-tracking group
+constexpr int G = 16;         // products per index-tracking group
 constexpr int TI = 4;         // rows per thread
 constexpr int TJ = 8;         // columns per thread
 constexpr int NT = 256;       // threads per workgroup
@@ -56,13 +58,16 @@ struct Params {
     float *c;
     int32_t *argmax;
     int32_t *argmin;
-    float *part;      // split-K partials: [split][4 or 2][N*M]
+    float *part;      // split-K partials: [split][3 or 2][N*M]: max, min, (group ids packed 16:16)
     int N, K, M;
     int tiles_n, tiles_m, splits, k_per_split;
     int vec_x, vec_w;  // 16-byte global loads are legal for x / w
+    int fast;          // the k-invariant 32-bit-offset staging path is legal
 };
 
 // First k in group g (ascending) whose product equals `target`; value recomputed from it.
+// The cost of this step is the number of cache lines each wave touches, not arithmetic, so the
+// G operands of each side are fetched with 16-byte loads when the layout allows it.
 template <int LAYOUT>
 __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, float target,
                                         float &val, int &idx)
@@ -72,11 +77,34 @@ __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, fl
     idx = kb < klast ? kb : klast;
     val = target;
     const float *xr = p.x + (int64_t)n * p.ldx;
+    float xv[G], wv[G];
+    const bool whole = kb + G <= p.K;
+    if (whole && p.vec_x) {
+#pragma unroll
+        for (int q = 0; q < G / 4; ++q) {
+            const float4 a = *reinterpret_cast<const float4 *>(xr + kb + q * 4);
+            xv[q * 4 + 0] = a.x; xv[q * 4 + 1] = a.y; xv[q * 4 + 2] = a.z; xv[q * 4 + 3] = a.w;
+        }
+    } else {
+#pragma unroll
+        for (int kk = 0; kk < G; ++kk) xv[kk] = xr[(kb + kk) < klast ? (kb + kk) : klast];
+    }
+    if (LAYOUT == MAM_W_MK && whole && p.vec_w) {
+        const float *wr = p.w + (int64_t)m * p.ldw + kb;
+#pragma unroll
+        for (int q = 0; q < G / 4; ++q) {
+            const float4 a = *reinterpret_cast<const float4 *>(wr + q * 4);
+            wv[q * 4 + 0] = a.x; wv[q * 4 + 1] = a.y; wv[q * 4 + 2] = a.z; wv[q * 4 + 3] = a.w;
+        }
+    } else {
+#pragma unroll
+        for (int kk = 0; kk < G; ++kk)
+            wv[kk] = load_w<LAYOUT>(p.w, p.ldw, (kb + kk) < klast ? (kb + kk) : klast, m);
+    }
 #pragma unroll
     for (int kk = G - 1; kk >= 0; --kk) {
-        const int k = (kb + kk) < klast ? (kb + kk) : klast;
-        const float prod = xr[k] * load_w<LAYOUT>(p.w, p.ldw, k, m);
-        if (prod == target) { idx = k; val = prod; }
+        const float prod = xv[kk] * wv[kk];
+        if (prod == target) { idx = (kb + kk) < klast ? (kb + kk) : klast; val = prod; }
     }
 }
 
@@ -117,11 +145,66 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
     }
 }
 
+// Stages one k-tile [k0, k0+KT) of X and W into LDS for any alignment and any ragged edge:
+// rows, columns and k beyond the problem are replaced by the last valid one.
+template <int LAYOUT>
+__device__ __forceinline__ void stage_tile_generic(const Params &p, float (*xs)[LDK], float (*ws)[LDK],
+                                                   int tid, int row0, int col0, int k0, int ke)
+{
+    const int kl = ke - 1;
+#pragma unroll
+    for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
+        const int e = tid + it * NT;
+        const int r = e >> 3, ch = e & 7;
+        const int row = (row0 + r) < p.N ? (row0 + r) : (p.N - 1);
+        const int k = k0 + ch * 4;
+        const float *src = p.x + (int64_t)row * p.ldx;
+        float4 v;
+        v.x = src[k < kl ? k : kl];
+        v.y = src[k + 1 < kl ? k + 1 : kl];
+        v.z = src[k + 2 < kl ? k + 2 : kl];
+        v.w = src[k + 3 < kl ? k + 3 : kl];
+        *reinterpret_cast<float4 *>(&xs[r][ch * 4]) = v;
+    }
+    if (LAYOUT == MAM_W_MK) {
+#pragma unroll
+        for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+            const int e = tid + it * NT;
+            const int r = e >> 3, ch = e & 7;
+            const int col = (col0 + r) < p.M ? (col0 + r) : (p.M - 1);
+            const int k = k0 + ch * 4;
+            const float *src = p.w + (int64_t)col * p.ldw;
+            float4 v;
+            v.x = src[k < kl ? k : kl];
+            v.y = src[k + 1 < kl ? k + 1 : kl];
+            v.z = src[k + 2 < kl ? k + 2 : kl];
+            v.w = src[k + 3 < kl ? k + 3 : kl];
+            *reinterpret_cast<float4 *>(&ws[r][ch * 4]) = v;
+        }
+    } else {
+#pragma unroll
+        for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+            const int e = tid + it * NT;
+            const int c4 = (e & 7) + ((e >> 8) << 3);
+            const int kk = (e >> 3) & 31;
+            const int k = (k0 + kk) < kl ? (k0 + kk) : kl;
+            const int mb = col0 + c4 * 4;
+            const int ml = p.M - 1;
+            const float *src = p.w + (int64_t)k * p.ldw;
+            ws[c4 * 4 + 0][kk] = src[mb < ml ? mb : ml];
+            ws[c4 * 4 + 1][kk] = src[mb + 1 < ml ? mb + 1 : ml];
+            ws[c4 * 4 + 2][kk] = src[mb + 2 < ml ? mb + 2 : ml];
+            ws[c4 * 4 + 3][kk] = src[mb + 3 < ml ? mb + 3 : ml];
+        }
+    }
+}
+
 template <int LAYOUT, bool ARGS>
 __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 {
-    __shared__ __attribute__((aligned(16))) float xs[BN][LDK];
-    __shared__ __attribute__((aligned(16))) float ws[BM][LDK];
+    __shared__ __attribute__((aligned(16))) float smem[(BN + BM) * LDK];
+    float (*xs)[LDK] = reinterpret_cast<float (*)[LDK]>(smem);
+    float (*ws)[LDK] = reinterpret_cast<float (*)[LDK]>(smem + BN * LDK);
 
     const int tid = threadIdx.x;
     const int tx = tid & 15;  // column lane: columns tx + 16*j
@@ -144,137 +227,127 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
     const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
 
     float vmax[TI][TJ], vmin[TI][TJ];
-    int gmax[TI][TJ], gmin[TI][TJ];
+    // group of the running max in bits 0..15, of the running min in bits 16..31, both counted
+    // from the first group of this workgroup's k range
+    uint32_t gsel[TI][TJ];
 #pragma unroll
     for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
             vmax[i][j] = -__builtin_inff();
             vmin[i][j] = __builtin_inff();
-            gmax[i][j] = kb / G;
-            gmin[i][j] = kb / G;
+            gsel[i][j] = 0u;
         }
 
-    for (int k0 = kb; k0 < ke; k0 += KT) {
-        // ---- stage the X tile: 64 rows x 8 chunks of 4 k ----
-        float4 xr[(BN * KT / 4) / NT];
+    // ---- fast staging path: 16-byte loads at offsets that do not depend on k ----
+    // x and (M,K) w: thread e covers row e/8, k chunk e%8; rows past the edge re-read the last
+    // row.  (K,M) w: thread covers k row (e/8)%32 and four columns; needs a full column tile.
+    const bool fast = p.fast && (LAYOUT == MAM_W_MK || col0 + BM <= p.M);
+    uint32_t xo[(BN * KT / 4) / NT], wo[(BM * KT / 4) / NT];
 #pragma unroll
-        for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
-            const int e = tid + it * NT;
+    for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
+        const int e = tid + it * NT;
+        const int r = e >> 3, ch = e & 7;
+        const int row = ((row0 + r) < p.N ? (row0 + r) : (p.N - 1)) - row0;
+        xo[it] = (uint32_t)(row * (int)p.ldx + ch * 4);
+    }
+#pragma unroll
+    for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+        const int e = tid + it * NT;
+        if (LAYOUT == MAM_W_MK) {
             const int r = e >> 3, ch = e & 7;
-            const int row = (row0 + r) < p.N ? (row0 + r) : (p.N - 1);
-            const int k = k0 + ch * 4;
-            const float *src = p.x + (int64_t)row * p.ldx;
-            if (p.vec_x && k + 3 < ke) {
-                xr[it] = *reinterpret_cast<const float4 *>(src + k);
-            } else {
-                const int kl = ke - 1;
-                xr[it].x = src[k < kl ? k : kl];
-                xr[it].y = src[k + 1 < kl ? k + 1 : kl];
-                xr[it].z = src[k + 2 < kl ? k + 2 : kl];
-                xr[it].w = src[k + 3 < kl ? k + 3 : kl];
-            }
+            const int col = ((col0 + r) < p.M ? (col0 + r) : (p.M - 1)) - col0;
+            wo[it] = (uint32_t)(col * (int)p.ldw + ch * 4);
+        } else {
+            const int c4 = (e & 7) + ((e >> 8) << 3);
+            const int kk = (e >> 3) & 31;
+            wo[it] = (uint32_t)(kk * (int)p.ldw + c4 * 4);
         }
-        // ---- stage the W tile ----
-        float4 wr[(BM * KT / 4) / NT];
-        if (LAYOUT == MAM_W_MK) {
+    }
+    const float *xbase = p.x + (int64_t)row0 * p.ldx;
+    const float *wbase = LAYOUT == MAM_W_MK ? p.w + (int64_t)col0 * p.ldw : p.w + col0;
+
+    for (int k0 = kb; k0 < ke; k0 += KT) {
+        if (fast && k0 + KT <= ke) {
+            const float *xt = xbase + k0;
+            const float *wt = LAYOUT == MAM_W_MK ? wbase + k0 : wbase + (int64_t)k0 * p.ldw;
+            float4 xr[(BN * KT / 4) / NT], wr[(BM * KT / 4) / NT];
+#pragma unroll
+            for (int it = 0; it < (BN * KT / 4) / NT; ++it)
+                xr[it] = *reinterpret_cast<const float4 *>(xt + xo[it]);
+#pragma unroll
+            for (int it = 0; it < (BM * KT / 4) / NT; ++it)
+                wr[it] = *reinterpret_cast<const float4 *>(wt + wo[it]);
+#pragma unroll
+            for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
+                const int e = tid + it * NT;
+                *reinterpret_cast<float4 *>(&xs[e >> 3][(e & 7) * 4]) = xr[it];
+            }
 #pragma unroll
             for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
                 const int e = tid + it * NT;
-                const int r = e >> 3, ch = e & 7;
-                const int col = (col0 + r) < p.M ? (col0 + r) : (p.M - 1);
-                const int k = k0 + ch * 4;
-                const float *src = p.w + (int64_t)col * p.ldw;
-                if (p.vec_w && k + 3 < ke) {
-                    wr[it] = *reinterpret_cast<const float4 *>(src + k);
+                if (LAYOUT == MAM_W_MK) {
+                    *reinterpret_cast<float4 *>(&ws[e >> 3][(e & 7) * 4]) = wr[it];
                 } else {
-                    const int kl = ke - 1;
-                    wr[it].x = src[k < kl ? k : kl];
-                    wr[it].y = src[k + 1 < kl ? k + 1 : kl];
-                    wr[it].z = src[k + 2 < kl ? k + 2 : kl];
-                    wr[it].w = src[k + 3 < kl ? k + 3 : kl];
+                    const int c4 = (e & 7) + ((e >> 8) << 3);
+                    const int kk = (e >> 3) & 31;
+                    ws[c4 * 4 + 0][kk] = wr[it].x;
+                    ws[c4 * 4 + 1][kk] = wr[it].y;
+                    ws[c4 * 4 + 2][kk] = wr[it].z;
+                    ws[c4 * 4 + 3][kk] = wr[it].w;
                 }
             }
         } else {
-            // (K, M) operand: rows of w are contiguous along m; 8 lanes fetch 128 bytes of
-            // one k, and the tile is transposed on the way into LDS.
-#pragma unroll
-            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
-                const int e = tid + it * NT;
-                const int c4 = (e & 7) + ((e >> 8) << 3);
-                const int kk = (e >> 3) & 31;
-                const int k = (k0 + kk) < ke ? (k0 + kk) : (ke - 1);
-                const int mb = col0 + c4 * 4;
-                const float *src = p.w + (int64_t)k * p.ldw;
-                if (p.vec_w && mb + 3 < p.M) {
-                    wr[it] = *reinterpret_cast<const float4 *>(src + mb);
-                } else {
-                    const int ml = p.M - 1;
-                    wr[it].x = src[mb < ml ? mb : ml];
-                    wr[it].y = src[mb + 1 < ml ? mb + 1 : ml];
-                    wr[it].z = src[mb + 2 < ml ? mb + 2 : ml];
-                    wr[it].w = src[mb + 3 < ml ? mb + 3 : ml];
-                }
-            }
-        }
-#pragma unroll
-        for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
-            const int e = tid + it * NT;
-            *reinterpret_cast<float4 *>(&xs[e >> 3][(e & 7) * 4]) = xr[it];
-        }
-        if (LAYOUT == MAM_W_MK) {
-#pragma unroll
-            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
-                const int e = tid + it * NT;
-                *reinterpret_cast<float4 *>(&ws[e >> 3][(e & 7) * 4]) = wr[it];
-            }
-        } else {
-#pragma unroll
-            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
-                const int e = tid + it * NT;
-                const int c4 = (e & 7) + ((e >> 8) << 3);
-                const int kk = (e >> 3) & 31;
-                ws[c4 * 4 + 0][kk] = wr[it].x;
-                ws[c4 * 4 + 1][kk] = wr[it].y;
-                ws[c4 * 4 + 2][kk] = wr[it].z;
-                ws[c4 * 4 + 3][kk] = wr[it].w;
-            }
+            stage_tile_generic<LAYOUT>(p, xs, ws, tid, row0, col0, k0, ke);
         }
         __syncthreads();
 
-        // ---- 4 groups of 8 k: 32 outputs x 8 products each ----
-#pragma unroll 2
-        for (int gg = 0; gg < KT / G; ++gg) {
-            const int g = k0 / G + gg;
-            float4 xv[TI][2];
+        // ---- 2 groups of 16 k: 32 outputs x 16 products each.  The two groups are unrolled
+        // so that the running extremes ping-pong between two register sets: the value before
+        // the group stays readable for the "did it improve" test without a copy. ----
 #pragma unroll
-            for (int i = 0; i < TI; ++i) {
-                xv[i][0] = *reinterpret_cast<const float4 *>(&xs[ty + 16 * i][gg * G]);
-                xv[i][1] = *reinterpret_cast<const float4 *>(&xs[ty + 16 * i][gg * G + 4]);
-            }
+        for (int gg = 0; gg < KT / G; ++gg) {
+            const uint32_t grel = (uint32_t)((k0 - kb) / G + gg);
+            float xv[TI][G];
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int q = 0; q < G / 4; ++q) {
+                    const float4 t = *reinterpret_cast<const float4 *>(&xs[ty + 16 * i][gg * G + q * 4]);
+                    xv[i][q * 4 + 0] = t.x; xv[i][q * 4 + 1] = t.y;
+                    xv[i][q * 4 + 2] = t.z; xv[i][q * 4 + 3] = t.w;
+                }
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                const float4 wa = *reinterpret_cast<const float4 *>(&ws[tx + 16 * j][gg * G]);
-                const float4 wb = *reinterpret_cast<const float4 *>(&ws[tx + 16 * j][gg * G + 4]);
+                float wv[G];
+#pragma unroll
+                for (int q = 0; q < G / 4; ++q) {
+                    const float4 t = *reinterpret_cast<const float4 *>(&ws[tx + 16 * j][gg * G + q * 4]);
+                    wv[q * 4 + 0] = t.x; wv[q * 4 + 1] = t.y;
+                    wv[q * 4 + 2] = t.z; wv[q * 4 + 3] = t.w;
+                }
 #pragma unroll
                 for (int i = 0; i < TI; ++i) {
-                    const float p0 = xv[i][0].x * wa.x, p1 = xv[i][0].y * wa.y;
-                    const float p2 = xv[i][0].z * wa.z, p3 = xv[i][0].w * wa.w;
-                    const float p4 = xv[i][1].x * wb.x, p5 = xv[i][1].y * wb.y;
-                    const float p6 = xv[i][1].z * wb.z, p7 = xv[i][1].w * wb.w;
-                    const float om = vmax[i][j];
-                    float hi = __builtin_fmaxf(__builtin_fmaxf(om, p0), p1);
-                    hi = __builtin_fmaxf(__builtin_fmaxf(hi, p2), p3);
-                    hi = __builtin_fmaxf(__builtin_fmaxf(hi, p4), p5);
-                    hi = __builtin_fmaxf(__builtin_fmaxf(hi, p6), p7);
-                    const float on = vmin[i][j];
-                    float lo = __builtin_fminf(__builtin_fminf(on, p0), p1);
-                    lo = __builtin_fminf(__builtin_fminf(lo, p2), p3);
-                    lo = __builtin_fminf(__builtin_fminf(lo, p4), p5);
-                    lo = __builtin_fminf(__builtin_fminf(lo, p6), p7);
+                    const float om = vmax[i][j], on = vmin[i][j];
+                    float hi = om, lo = on;
+#pragma unroll
+                    for (int q = 0; q < G; q += 2) {
+                        const float a = xv[i][q] * wv[q], b = xv[i][q + 1] * wv[q + 1];
+                        hi = __builtin_fmaxf(__builtin_fmaxf(hi, a), b);   // v_max3_f32
+                        lo = __builtin_fminf(__builtin_fminf(lo, a), b);   // v_min3_f32
+                    }
                     if (ARGS) {
-                        gmax[i][j] = (hi > om) ? g : gmax[i][j];
-                        gmin[i][j] = (lo < on) ? g : gmin[i][j];
+                        // gsel.lo16 = (hi > om) ? grel : gsel.lo16 ; gsel.hi16 likewise for the min.
+                        // One compare and one sub-dword conditional move per extreme: the select
+                        // picks a 16-bit word of each source and writes one word of gsel.
+                        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+                            "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE "
+                            "src0_sel:WORD_0 src1_sel:WORD_0"
+                            : "+v"(gsel[i][j]) : "v"(hi), "v"(om), "v"(grel) : "vcc");
+                        asm("v_cmp_lt_f32 vcc, %1, %2\n\t"
+                            "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE "
+                            "src0_sel:WORD_1 src1_sel:WORD_0"
+                            : "+v"(gsel[i][j]) : "v"(lo), "v"(on), "v"(grel) : "vcc");
                     }
                     vmax[i][j] = hi;
                     vmin[i][j] = lo;
@@ -285,18 +358,38 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
     }
 
     // ---- epilogue ----
+    const int g0 = kb / G;
     if (p.splits == 1) {
+        // The tiles in LDS are dead (the k loop ended on a barrier).  Each thread parks one row
+        // of its results in its own LDS slots so that the index resolution can be a rolled loop
+        // over j: one copy of the code per row instead of 32, and no register array indexed at
+        // run time.
+        static_assert(3 * TJ * NT <= (BN + BM) * LDK, "result stash does not fit the tile buffer");
+        float *stash = smem + tid;
 #pragma unroll
-        for (int i = 0; i < TI; ++i)
+        for (int i = 0; i < TI; ++i) {
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                const int n = row0 + ty + 16 * i, m = col0 + tx + 16 * j;
-                if (n < p.N && m < p.M)
-                    finish<LAYOUT, ARGS>(p, n, m, vmax[i][j], vmin[i][j], gmax[i][j], gmin[i][j]);
+                stash[(0 * TJ + j) * NT] = vmax[i][j];
+                stash[(1 * TJ + j) * NT] = vmin[i][j];
+                stash[(2 * TJ + j) * NT] = __uint_as_float(gsel[i][j]);
             }
+            const int n = row0 + ty + 16 * i;
+            if (n < p.N) {
+#pragma unroll 1
+                for (int j = 0; j < TJ; ++j) {
+                    const int m = col0 + tx + 16 * j;
+                    if (m < p.M) {
+                        const uint32_t gs = __float_as_uint(stash[(2 * TJ + j) * NT]);
+                        finish<LAYOUT, ARGS>(p, n, m, stash[(0 * TJ + j) * NT], stash[(1 * TJ + j) * NT],
+                                             g0 + (int)(gs & 0xffffu), g0 + (int)(gs >> 16));
+                    }
+                }
+            }
+        }
     } else {
         const int64_t nm = (int64_t)p.N * p.M;
-        float *base = p.part + (int64_t)split * (ARGS ? 4 : 2) * nm;
+        float *base = p.part + (int64_t)split * (ARGS ? 3 : 2) * nm;
 #pragma unroll
         for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -306,10 +399,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
                     const int64_t o = (int64_t)n * p.M + m;
                     base[o] = vmax[i][j];
                     base[nm + o] = vmin[i][j];
-                    if (ARGS) {
-                        base[2 * nm + o] = __int_as_float(gmax[i][j]);
-                        base[3 * nm + o] = __int_as_float(gmin[i][j]);
-                    }
+                    if (ARGS) base[2 * nm + o] = __uint_as_float(gsel[i][j]);
                 }
             }
     }
@@ -323,23 +413,27 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
     const int64_t nm = (int64_t)p.N * p.M;
     const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (o >= nm) return;
-    const int stride = ARGS ? 4 : 2;
+    const int stride = ARGS ? 3 : 2;
+    const int gps = p.k_per_split / G;   // groups per split
     float vmax = p.part[o], vmin = p.part[nm + o];
     int gmax = 0, gmin = 0;
     if (ARGS) {
-        gmax = __float_as_int(p.part[2 * nm + o]);
-        gmin = __float_as_int(p.part[3 * nm + o]);
+        const int pk = __float_as_int(p.part[2 * nm + o]);
+        gmax = pk & 0xffff;
+        gmin = (pk >> 16) & 0xffff;
     }
     for (int s = 1; s < p.splits; ++s) {
         const float *base = p.part + (int64_t)s * stride * nm;
         const float hi = base[o], lo = base[nm + o];
+        int pk = 0;
+        if (ARGS) pk = __float_as_int(base[2 * nm + o]);
         if (hi > vmax) {
             vmax = hi;
-            if (ARGS) gmax = __float_as_int(base[2 * nm + o]);
+            gmax = s * gps + (pk & 0xffff);
         }
         if (lo < vmin) {
             vmin = lo;
-            if (ARGS) gmin = __float_as_int(base[3 * nm + o]);
+            gmin = s * gps + ((pk >> 16) & 0xffff);
         }
     }
     const int n = (int)(o / p.M), m = (int)(o - (int64_t)n * p.M);
@@ -356,14 +450,17 @@ static int choose_splits(int64_t N, int64_t K, int64_t M)
     const int64_t max_by_k = K / (8 * KT);  // keep at least 256 k per split
     if (s > max_by_k) s = max_by_k;
     if (s > MAX_SPLITS) s = MAX_SPLITS;
-    return s < 1 ? 1 : (int)s;
+    if (s < 1) s = 1;
+    // partial group ids are 16-bit offsets within a split
+    if (s > 1 && ceil_div(ceil_div(K, s), KT) * KT / G > 65536) s = 1;
+    return (int)s;
 }
 
 static size_t workspace_bytes(int64_t N, int64_t K, int64_t M, bool args)
 {
     const int s = choose_splits(N, K, M);
     if (s == 1) return 0;
-    return (size_t)s * (args ? 4 : 2) * (size_t)N * (size_t)M * sizeof(float);
+    return (size_t)s * (args ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float);
 }
 
 template <bool ARGS>
@@ -394,7 +491,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     p.splits = (int)ceil_div(K, p.k_per_split);
     p.part = nullptr;
     if (p.splits > 1) {
-        const size_t need = (size_t)p.splits * (ARGS ? 4 : 2) * (size_t)N * (size_t)M * sizeof(float);
+        const size_t need = (size_t)p.splits * (ARGS ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float);
         if (!workspace || workspace_size < need)
             return fail(MAM_ERR_WORKSPACE, "forward needs %zu workspace bytes, got %zu", need,
                         workspace ? workspace_size : (size_t)0);
@@ -402,6 +499,12 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     }
     p.vec_x = (ldx % 4 == 0) && ((uintptr_t)x % 16 == 0);
     p.vec_w = (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0);
+    // the fast staging path addresses a tile with 32-bit element offsets from the tile base
+    const int64_t w_rows = (w_layout == MAM_W_MK) ? fwd::BM : fwd::KT;
+    p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30));
+    // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
+    if ((int64_t)p.k_per_split / G > 65536)
+        return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds %d per K range", (long long)K, 65536 * G);
 
     const int64_t nblk = (int64_t)p.tiles_n * p.tiles_m * p.splits;
     if (nblk > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "too many tiles");

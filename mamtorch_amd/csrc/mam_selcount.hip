@@ -9,7 +9,7 @@
 // set bits and applies plain read-modify-writes to its own rows: the counters are touched only
 // where something was picked, and no global atomics are needed.
 //
-// MAM_COUNT_HITS counts every pick (global int atomics; fire-and-forget).
+// MAM_COUNT_HITS counts every pick with the same ownership scheme and LDS counters.
 #include "mam_common.h"
 
 namespace mam {
@@ -17,18 +17,76 @@ namespace selcount {
 
 constexpr int NT = 256;
 
-__global__ __launch_bounds__(NT) void hits_kernel(const int32_t *__restrict__ argmax,
-                                                  const int32_t *__restrict__ argmin,
-                                                  int32_t *__restrict__ max_count,
-                                                  int32_t *__restrict__ min_count, int64_t NM, int M,
-                                                  int K)
+// Hit counting: a workgroup owns R neurons x kc columns of both counters.  Picks are counted in
+// LDS words holding two 16-bit counters (low half: argmax hits, high half: argmin hits; the batch
+// is walked in chunks of 32768 rows so that neither half overflows), then only the cells that
+// were hit are read-modify-written in HBM.
+constexpr int NT_H = 512;
+constexpr int ROWS_PER_PASS = 32768;
+
+__global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ argmax,
+                                                    const int32_t *__restrict__ argmin,
+                                                    int32_t *__restrict__ max_count,
+                                                    int32_t *__restrict__ min_count, int N, int M,
+                                                    int K, int log2r, int kc, int vec)
 {
-    const int64_t o = (int64_t)blockIdx.x * NT + threadIdx.x;
-    if (o >= NM) return;
-    const int m = (int)(o % M);
-    const int a1 = argmax[o], a2 = argmin[o];
-    if ((unsigned)a1 < (unsigned)K) atomicAdd(&max_count[(int64_t)m * K + a1], 1);
-    if ((unsigned)a2 < (unsigned)K) atomicAdd(&min_count[(int64_t)m * K + a2], 1);
+    extern __shared__ uint32_t cnt[];  // [R][kc]
+    const int tid = threadIdx.x;
+    const int R = 1 << log2r;
+    const int m0 = xcd_remap(blockIdx.x, gridDim.x) * R;
+    const int k0 = blockIdx.y * kc;
+    const int rn = (M - m0) < R ? (M - m0) : R;
+    const int kn = (K - k0) < kc ? (K - k0) : kc;
+    for (int n0 = 0; n0 < N; n0 += ROWS_PER_PASS) {
+        const int nn = (N - n0) < ROWS_PER_PASS ? (N - n0) : ROWS_PER_PASS;
+        for (int i = tid; i < R * kc; i += NT_H) cnt[i] = 0u;
+        __syncthreads();
+        const int pairs = nn << log2r;
+        for (int pi = tid; pi < pairs; pi += NT_H) {
+            const int n = n0 + (pi >> log2r), r = pi & (R - 1);
+            if (r >= rn) continue;
+            const int64_t o = (int64_t)n * M + m0 + r;
+            const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
+            if ((unsigned)a1 < (unsigned)kn) atomicAdd(&cnt[r * kc + a1], 1u);
+            if ((unsigned)a2 < (unsigned)kn) atomicAdd(&cnt[r * kc + a2], 0x10000u);
+        }
+        __syncthreads();
+        // Stream the slab back: 4 cells per lane, whole 16-byte chunks skipped when nothing in
+        // them was hit.  At training batch sizes nearly every cache line holds a hit, so this is
+        // a coalesced read-modify-write of the slab; at small N*M it degenerates to a sparse one.
+        if (vec) {
+            const int q = kn >> 2;
+            for (int e = tid; e < rn * q; e += NT_H) {
+                const int r = e / q, c4 = e - r * q;
+                const uint4 v = *reinterpret_cast<const uint4 *>(&cnt[r * kc + c4 * 4]);
+                if ((v.x | v.y | v.z | v.w) == 0u) continue;
+                const int64_t cell = (int64_t)(m0 + r) * K + k0 + c4 * 4;
+                if ((v.x | v.y | v.z | v.w) & 0xffffu) {
+                    int4 a = *reinterpret_cast<int4 *>(max_count + cell);
+                    a.x += (int)(v.x & 0xffffu); a.y += (int)(v.y & 0xffffu);
+                    a.z += (int)(v.z & 0xffffu); a.w += (int)(v.w & 0xffffu);
+                    *reinterpret_cast<int4 *>(max_count + cell) = a;
+                }
+                if ((v.x | v.y | v.z | v.w) >> 16) {
+                    int4 a = *reinterpret_cast<int4 *>(min_count + cell);
+                    a.x += (int)(v.x >> 16); a.y += (int)(v.y >> 16);
+                    a.z += (int)(v.z >> 16); a.w += (int)(v.w >> 16);
+                    *reinterpret_cast<int4 *>(min_count + cell) = a;
+                }
+            }
+        } else {
+            for (int e = tid; e < rn * kn; e += NT_H) {
+                const int r = e / kn, kk = e - r * kn;
+                const uint32_t v = cnt[r * kc + kk];
+                if (v) {
+                    const int64_t cell = (int64_t)(m0 + r) * K + k0 + kk;
+                    if (v & 0xffffu) max_count[cell] += (int)(v & 0xffffu);
+                    if (v >> 16) min_count[cell] += (int)(v >> 16);
+                }
+            }
+        }
+        __syncthreads();
+    }
 }
 
 __global__ __launch_bounds__(NT) void reference_kernel(const int32_t *__restrict__ argmax,
@@ -67,6 +125,15 @@ __global__ __launch_bounds__(NT) void reference_kernel(const int32_t *__restrict
     }
 }
 
+static int lds_budget_words(const void *kernel)
+{
+    constexpr int kWant = 128 * 1024;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kWant) == hipSuccess)
+        return kWant / 4;
+    (void)hipGetLastError();
+    return 64 * 1024 / 4;
+}
+
 }  // namespace selcount
 }  // namespace mam
 
@@ -85,10 +152,17 @@ extern "C" int mam_selection_count(const int32_t *argmax, const int32_t *argmin,
         return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (mode == MAM_COUNT_HITS) {
-        const int64_t nm = N * M;
-        hipLaunchKernelGGL(selcount::hits_kernel, dim3((unsigned)ceil_div(nm, selcount::NT)),
-                           dim3(selcount::NT), 0, st, argmax, argmin, max_count, min_count, nm, (int)M,
-                           (int)K);
+        static const int budget = selcount::lds_budget_words((const void *)selcount::hits_kernel);
+        const int log2r = 3;
+        const int R = 1 << log2r;
+        int kc = budget / R;
+        if (K < kc) kc = (int)((K + 3) / 4 * 4);
+        const int64_t ktiles = ceil_div(K, kc);
+        const int vec = (K % 4 == 0) && ((uintptr_t)max_count % 16 == 0) && ((uintptr_t)min_count % 16 == 0);
+        if (ktiles > 65535) return fail(MAM_ERR_UNSUPPORTED, "K too large for the selection-count grid");
+        hipLaunchKernelGGL(selcount::hits_kernel, dim3((unsigned)ceil_div(M, R), (unsigned)ktiles),
+                           dim3(selcount::NT_H), (size_t)R * kc * 4, st, argmax, argmin, max_count,
+                           min_count, (int)N, (int)M, (int)K, log2r, kc, vec);
         return check_launch("selcount::hits_kernel");
     }
     const int words = (int)ceil_div(K, 32);

@@ -37,8 +37,8 @@ def test_workspace_queries_are_pure_host_calls():
     l = capi.lib()
     assert l.mam_fc_forward_workspace(12608, 768, 3072) == 0          # enough tiles: no split-K
     ws = l.mam_fc_forward_workspace(256, 4096, 4096)
-    assert ws > 0 and ws % (256 * 4096 * 16) == 0                     # splits x (2 values + 2 groups) x N*M x 4 B
-    assert l.mam_fc_forward_values_workspace(256, 4096, 4096) * 2 == ws
+    assert ws > 0 and ws % (256 * 4096 * 12) == 0                     # splits x (max, min, packed groups) x N*M x 4 B
+    assert l.mam_fc_forward_values_workspace(256, 4096, 4096) * 3 == ws * 2
     assert l.mam_fc_forward_workspace(0, 5, 5) == 0
 
 
