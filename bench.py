@@ -65,8 +65,9 @@ def cpu_baseline(torch, x, w, g, budget_s):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=300,
+                    help="untimed steps; the GPU clock needs ~100 launches to ramp up")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     args = ap.parse_args()
     if args.gpus != 1:

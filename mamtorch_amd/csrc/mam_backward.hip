@@ -10,8 +10,9 @@
 //
 //   x_grad : one workgroup per batch row n; histogram over k (chunked when K floats exceed LDS).
 //   w_grad : one workgroup per R consecutive output neurons x KC consecutive k.  For the (M,K)
-//            layout R = 8 so a slab is 8 whole rows of the weight gradient; for the (K,M) layout
-//            R = 32 so that every stored row segment is 128 bytes.
+//            layout R = 4 so a slab is 4 whole rows of the weight gradient (64 KiB: two
+//            workgroups per CU); for the (K,M) layout R = 32 so that every stored row segment is
+//            128 bytes.
 //
 // Each term is one fp32 product (operand of the reference's atomicAdd); only the order of the
 // fp32 additions differs from the reference, which is itself unordered.
@@ -44,11 +45,30 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
         const int kn = (K - k0) < kc ? (K - k0) : kc;
         for (int i = tid; i < kn; i += NT_X) hist[i] = 0.0f;
         __syncthreads();
-        for (int m = tid; m < M; m += NT_X) {
-            const float g = g_row[m];
-            const int a1 = amax_row[m] - k0, a2 = amin_row[m] - k0;
-            if ((unsigned)a1 < (unsigned)kn) lds_add(&hist[a1], load_w<LAYOUT>(w, ldw, a1 + k0, m) * g);
-            if ((unsigned)a2 < (unsigned)kn) lds_add(&hist[a2], load_w<LAYOUT>(w, ldw, a2 + k0, m) * g);
+        // four outputs per thread and trip: all index loads, then all weight gathers, then the
+        // LDS adds, so that the gather latencies overlap instead of adding up
+        for (int mb = tid; mb < M; mb += 4 * NT_X) {
+            float g[4], wv1[4], wv2[4];
+            int a1[4], a2[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int m = mb + u * NT_X;
+                const bool ok = m < M;
+                g[u] = ok ? g_row[m] : 0.0f;
+                a1[u] = ok ? amax_row[m] - k0 : -1;
+                a2[u] = ok ? amin_row[m] - k0 : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int m = mb + u * NT_X;
+                wv1[u] = (unsigned)a1[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a1[u] + k0, m) : 0.0f;
+                wv2[u] = (unsigned)a2[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a2[u] + k0, m) : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if ((unsigned)a1[u] < (unsigned)kn) lds_add(&hist[a1[u]], wv1[u] * g[u]);
+                if ((unsigned)a2[u] < (unsigned)kn) lds_add(&hist[a2[u]], wv2[u] * g[u]);
+            }
         }
         __syncthreads();
         float *dst = x_grad + (int64_t)n * K + k0;
@@ -61,7 +81,8 @@ template <int LAYOUT>
 __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    float *__restrict__ w_grad, int N, int K, int M, int log2r, int kc, int vec_out)
+    float *__restrict__ w_grad, int N, int K, int M, int log2r, int kc, int vec_out,
+    int vec_in)
 {
     extern __shared__ float hist[];
     const int tid = threadIdx.x;
@@ -77,18 +98,50 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
         *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
 
-    const int64_t pairs = (int64_t)N << log2r;
-    for (int64_t pi = tid; pi < pairs; pi += NT_W) {
-        const int n = (int)(pi >> log2r), r = (int)(pi & (R - 1));
-        if (r >= rn) continue;
-        const int64_t o = (int64_t)n * M + m0 + r;
-        const float g = grad[o];
-        const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
-        const float *xr = x + (int64_t)n * ldx + k0;
-        if ((unsigned)a1 < (unsigned)kn)
-            lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r], xr[a1] * g);
-        if ((unsigned)a2 < (unsigned)kn)
-            lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r], xr[a2] * g);
+    if (vec_in && rn == R) {
+        // a thread takes 4 consecutive neurons of one batch row: three 16-byte loads, then the
+        // eight x gathers (all from one 4*K-byte row), then the LDS adds
+        const int qpr = R >> 2;   // quads per row
+        const int64_t items = (int64_t)N * qpr;
+        for (int64_t it = tid; it < items; it += NT_W) {
+            const int n = (int)(it / qpr), r0 = (int)(it - (int64_t)n * qpr) * 4;
+            const int64_t o = (int64_t)n * M + m0 + r0;
+            const float4 g = *reinterpret_cast<const float4 *>(grad + o);
+            const int4 i1 = *reinterpret_cast<const int4 *>(argmax + o);
+            const int4 i2 = *reinterpret_cast<const int4 *>(argmin + o);
+            const float gv[4] = {g.x, g.y, g.z, g.w};
+            const int a1[4] = {i1.x - k0, i1.y - k0, i1.z - k0, i1.w - k0};
+            const int a2[4] = {i2.x - k0, i2.y - k0, i2.z - k0, i2.w - k0};
+            const float *xr = x + (int64_t)n * ldx + k0;
+            float x1[4], x2[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                x1[u] = (unsigned)a1[u] < (unsigned)kn ? xr[a1[u]] : 0.0f;
+                x2[u] = (unsigned)a2[u] < (unsigned)kn ? xr[a2[u]] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int r = r0 + u;
+                if ((unsigned)a1[u] < (unsigned)kn)
+                    lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a1[u] : (a1[u] << log2r) + r], x1[u] * gv[u]);
+                if ((unsigned)a2[u] < (unsigned)kn)
+                    lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a2[u] : (a2[u] << log2r) + r], x2[u] * gv[u]);
+            }
+        }
+    } else {
+        const int64_t pairs = (int64_t)N << log2r;
+        for (int64_t pi = tid; pi < pairs; pi += NT_W) {
+            const int n = (int)(pi >> log2r), r = (int)(pi & (R - 1));
+            if (r >= rn) continue;
+            const int64_t o = (int64_t)n * M + m0 + r;
+            const float g = grad[o];
+            const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
+            const float *xr = x + (int64_t)n * ldx + k0;
+            if ((unsigned)a1 < (unsigned)kn)
+                lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r], xr[a1] * g);
+            if ((unsigned)a2 < (unsigned)kn)
+                lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r], xr[a2] * g);
+        }
     }
     __syncthreads();
 
@@ -141,17 +194,22 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         if (rc != MAM_OK) return rc;
     }
     if (w_grad) {
-        static const int budget = lds_budget_floats((const void *)mam_bwd_w_kernel<LAYOUT>);
-        const int log2r = LAYOUT == MAM_W_MK ? 3 : 5;
+        // (M,K): 4 whole-K rows in 64 KiB, so two workgroups share a CU and one's scatter phase
+        // overlaps the other's store phase.  (K,M): 32 columns x 1024 k in 128 KiB.
+        static const int big = lds_budget_floats((const void *)mam_bwd_w_kernel<LAYOUT>);
+        const int log2r = LAYOUT == MAM_W_MK ? 2 : 5;
         const int R = 1 << log2r;
+        const int budget = LAYOUT == MAM_W_MK ? 64 * 1024 / 4 : big;
         int kc = budget / R;
         if (K < kc) kc = (int)((K + 3) / 4 * 4);
         const int64_t mtiles = ceil_div(M, R), ktiles = ceil_div(K, kc);
         if (ktiles > 65535) return fail(MAM_ERR_UNSUPPORTED, "K too large for the w_grad grid");
         const int vec_out = (K % 4 == 0) && ((uintptr_t)w_grad % 16 == 0);
+        const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
+                           ((uintptr_t)argmin % 16 == 0);
         hipLaunchKernelGGL((mam_bwd_w_kernel<LAYOUT>), dim3((unsigned)mtiles, (unsigned)ktiles),
                            dim3(NT_W), (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax,
-                           argmin, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out);
+                           argmin, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out, vec_in);
         rc = check_launch("mam_bwd_w_kernel");
     }
     return rc;

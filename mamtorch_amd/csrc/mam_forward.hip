@@ -199,16 +199,128 @@ __device__ __forceinline__ void stage_tile_generic(const Params &p, float (*xs)[
     }
 }
 
+// Stages one full, 16-byte-aligned k-tile of the (K, M) operand through registers: 8 lanes fetch
+// 128 bytes of one k row, and the tile is transposed on the way into LDS.
+__device__ __forceinline__ void stage_w_km_fast(const float *wt, float (*ws)[LDK], int tid,
+                                                const uint32_t (&wo)[(BM * KT / 4) / NT])
+{
+    float4 wr[(BM * KT / 4) / NT];
+#pragma unroll
+    for (int it = 0; it < (BM * KT / 4) / NT; ++it) wr[it] = *reinterpret_cast<const float4 *>(wt + wo[it]);
+#pragma unroll
+    for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+        const int e = tid + it * NT;
+        const int c4 = (e & 7) + ((e >> 8) << 3);
+        const int kk = (e >> 3) & 31;
+        ws[c4 * 4 + 0][kk] = wr[it].x;
+        ws[c4 * 4 + 1][kk] = wr[it].y;
+        ws[c4 * 4 + 2][kk] = wr[it].z;
+        ws[c4 * 4 + 3][kk] = wr[it].w;
+    }
+}
+
+// One wave-level direct-to-LDS load moves 64 x 16 bytes into 1 KiB of consecutive LDS.  A tile
+// (X rows then W rows, 9 16-byte slots per row: 8 of data, 1 of padding) is exactly 27 such loads,
+// the first 9 of them X; wave w issues loads w, w+4, ...  No register holds the data in flight.
+constexpr int TILE_FLOATS = (BN + BM) * LDK;
+constexpr int DMA_INSTR = TILE_FLOATS / 4 / 64;
+constexpr int DMA_X_INSTR = BN * LDK / 4 / 64;
+constexpr int DMA_PER_WAVE = (DMA_INSTR + NT / 64 - 1) / (NT / 64);
+static_assert(TILE_FLOATS % 256 == 0 && (BN * LDK) % 256 == 0, "tile must be whole wave-level loads");
+
+// Per-lane source offsets of a wave's loads live in LDS ([load][thread]): they are needed once
+// per tile, and a register spilled to scratch would be reloaded through the same counter that
+// tracks the loads in flight.
+__device__ __forceinline__ void dma_tile(const float *xt, const float *wt, float *tile, int wave,
+                                         const uint32_t *doff, bool x_only)
+{
+#pragma unroll
+    for (int t = 0; t < DMA_PER_WAVE; ++t) {
+        // every wave issues DMA_PER_WAVE loads; the one past the end repeats the last load
+        int inst = wave + (NT / 64) * t;
+        inst = inst < DMA_INSTR ? inst : DMA_INSTR - 1;
+        if (x_only && t * (NT / 64) >= DMA_X_INSTR) break;
+        if (x_only) inst = inst < DMA_X_INSTR ? inst : DMA_X_INSTR - 1;
+        const float *src = (inst < DMA_X_INSTR ? xt : wt) + doff[t * NT];
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void *)src,
+            (__attribute__((address_space(3))) void *)(tile + inst * 256), 16, 0, 0);
+    }
+}
+
+// 2 groups of 16 k from one staged tile: 32 outputs x 16 products each.  The two groups are
+// unrolled so that the running extremes ping-pong between two register sets: the value before
+// the group stays readable for the "did it improve" test without a copy.
+template <bool ARGS>
+__device__ __forceinline__ void compute_tile(const float *tile, int tx, int ty, uint32_t grel0,
+                                             float (&vmax)[TI][TJ], float (&vmin)[TI][TJ],
+                                             uint32_t (&gsel)[TI][TJ])
+{
+    const float (*xs)[LDK] = reinterpret_cast<const float (*)[LDK]>(tile);
+    const float (*ws)[LDK] = reinterpret_cast<const float (*)[LDK]>(tile + BN * LDK);
+#pragma unroll
+    for (int gg = 0; gg < KT / G; ++gg) {
+        const uint32_t grel = grel0 + gg;
+        float xv[TI][G];
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int q = 0; q < G / 4; ++q) {
+                const float4 t = *reinterpret_cast<const float4 *>(&xs[ty + 16 * i][gg * G + q * 4]);
+                xv[i][q * 4 + 0] = t.x; xv[i][q * 4 + 1] = t.y;
+                xv[i][q * 4 + 2] = t.z; xv[i][q * 4 + 3] = t.w;
+            }
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            float wv[G];
+#pragma unroll
+            for (int q = 0; q < G / 4; ++q) {
+                const float4 t = *reinterpret_cast<const float4 *>(&ws[tx + 16 * j][gg * G + q * 4]);
+                wv[q * 4 + 0] = t.x; wv[q * 4 + 1] = t.y;
+                wv[q * 4 + 2] = t.z; wv[q * 4 + 3] = t.w;
+            }
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                const float om = vmax[i][j], on = vmin[i][j];
+                float hi = om, lo = on;
+#pragma unroll
+                for (int q = 0; q < G; q += 2) {
+                    const float a = xv[i][q] * wv[q], b = xv[i][q + 1] * wv[q + 1];
+                    hi = __builtin_fmaxf(__builtin_fmaxf(hi, a), b);   // v_max3_f32
+                    lo = __builtin_fminf(__builtin_fminf(lo, a), b);   // v_min3_f32
+                }
+                if (ARGS) {
+                    // gsel.lo16 = (hi > om) ? grel : gsel.lo16 ; gsel.hi16 likewise for the min.
+                    // One compare and one sub-dword conditional move per extreme: the select
+                    // picks a 16-bit word of each source and writes one word of gsel.
+                    asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
+                        "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE "
+                        "src0_sel:WORD_0 src1_sel:WORD_0"
+                        : "+v"(gsel[i][j]) : "v"(hi), "v"(om), "v"(grel) : "vcc");
+                    asm("v_cmp_lt_f32 vcc, %1, %2\n\t"
+                        "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE "
+                        "src0_sel:WORD_1 src1_sel:WORD_0"
+                        : "+v"(gsel[i][j]) : "v"(lo), "v"(on), "v"(grel) : "vcc");
+                }
+                vmax[i][j] = hi;
+                vmin[i][j] = lo;
+            }
+        }
+    }
+}
+
 template <int LAYOUT, bool ARGS>
 __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 {
-    __shared__ __attribute__((aligned(16))) float smem[(BN + BM) * LDK];
-    float (*xs)[LDK] = reinterpret_cast<float (*)[LDK]>(smem);
-    float (*ws)[LDK] = reinterpret_cast<float (*)[LDK]>(smem + BN * LDK);
+    // Two tile buffers as two separate arrays: the compiler can then see that loads in flight
+    // into one never alias reads of the other, and lets them overlap.
+    __shared__ __attribute__((aligned(16))) float tile_a[TILE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float tile_b[TILE_FLOATS];
 
     const int tid = threadIdx.x;
     const int tx = tid & 15;  // column lane: columns tx + 16*j
     const int ty = tid >> 4;  // row lane:    rows    ty + 16*i
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     // ---- which tile: XCD-aware, then row tiles grouped under one W panel ----
     const int logical = xcd_remap(blockIdx.x, gridDim.x);
@@ -225,6 +337,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
     const int row0 = tn * BN, col0 = tm * BM;
     const int kb = split * p.k_per_split;
     const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
+    const int ntiles = (ke - kb + KT - 1) / KT;
 
     float vmax[TI][TJ], vmin[TI][TJ];
     // group of the running max in bits 0..15, of the running min in bits 16..31, both counted
@@ -239,121 +352,74 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
             gsel[i][j] = 0u;
         }
 
-    // ---- fast staging path: 16-byte loads at offsets that do not depend on k ----
-    // x and (M,K) w: thread e covers row e/8, k chunk e%8; rows past the edge re-read the last
-    // row.  (K,M) w: thread covers k row (e/8)%32 and four columns; needs a full column tile.
+    // ---- staging ----
+    // Full, aligned tiles take a fast path whose per-thread source offsets do not depend on k
+    // (rows / columns past the edge re-read the last valid one).  For x and an (M,K) w that
+    // path is direct-to-LDS and runs one tile ahead of the arithmetic; a (K,M) w goes through
+    // registers because it has to be transposed, and needs a full column tile.  Everything
+    // else (ragged k tail, unaligned views) takes the generic path.
     const bool fast = p.fast && (LAYOUT == MAM_W_MK || col0 + BM <= p.M);
-    uint32_t xo[(BN * KT / 4) / NT], wo[(BM * KT / 4) / NT];
+    const float *xbase = p.x + (int64_t)row0 * p.ldx;
+    const float *wbase = LAYOUT == MAM_W_MK ? p.w + (int64_t)col0 * p.ldw : p.w + col0;
+    __shared__ uint32_t doff_s[DMA_PER_WAVE * NT];
+    const uint32_t *doff = doff_s + tid;
 #pragma unroll
-    for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
-        const int e = tid + it * NT;
-        const int r = e >> 3, ch = e & 7;
-        const int row = ((row0 + r) < p.N ? (row0 + r) : (p.N - 1)) - row0;
-        xo[it] = (uint32_t)(row * (int)p.ldx + ch * 4);
-    }
-#pragma unroll
-    for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
-        const int e = tid + it * NT;
-        if (LAYOUT == MAM_W_MK) {
-            const int r = e >> 3, ch = e & 7;
-            const int col = ((col0 + r) < p.M ? (col0 + r) : (p.M - 1)) - col0;
-            wo[it] = (uint32_t)(col * (int)p.ldw + ch * 4);
+    for (int t = 0; t < DMA_PER_WAVE; ++t) {
+        int inst = wave + (NT / 64) * t;
+        inst = inst < DMA_INSTR ? inst : DMA_INSTR - 1;
+        if (LAYOUT == MAM_W_KM) inst = inst < DMA_X_INSTR ? inst : DMA_X_INSTR - 1;
+        const int slot = inst * 64 + (tid & 63);
+        const int row = slot / (LDK / 4), pos = slot % (LDK / 4);
+        const int ch = pos < KT / 4 ? pos : KT / 4 - 1;   // the padding slot re-reads the last chunk
+        uint32_t off;
+        if (row < BN) {
+            const int r = ((row0 + row) < p.N ? (row0 + row) : (p.N - 1)) - row0;
+            off = (uint32_t)(r * (int)p.ldx + ch * 4);
         } else {
+            const int c = ((col0 + row - BN) < p.M ? (col0 + row - BN) : (p.M - 1)) - col0;
+            off = (uint32_t)(c * (int)p.ldw + ch * 4);
+        }
+        doff_s[t * NT + tid] = off;
+    }
+    uint32_t wo[(BM * KT / 4) / NT];   // (K,M) register path only
+    if (LAYOUT == MAM_W_KM) {
+#pragma unroll
+        for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
+            const int e = tid + it * NT;
             const int c4 = (e & 7) + ((e >> 8) << 3);
             const int kk = (e >> 3) & 31;
             wo[it] = (uint32_t)(kk * (int)p.ldw + c4 * 4);
         }
     }
-    const float *xbase = p.x + (int64_t)row0 * p.ldx;
-    const float *wbase = LAYOUT == MAM_W_MK ? p.w + (int64_t)col0 * p.ldw : p.w + col0;
 
-    for (int k0 = kb; k0 < ke; k0 += KT) {
+    // stage tile `t` into `dst`; returns after the loads are ISSUED (direct-to-LDS) or DONE
+    auto stage = [&](float *dst, int t) {
+        const int k0 = kb + t * KT;
+        float (*xs)[LDK] = reinterpret_cast<float (*)[LDK]>(dst);
+        float (*ws)[LDK] = reinterpret_cast<float (*)[LDK]>(dst + BN * LDK);
         if (fast && k0 + KT <= ke) {
-            const float *xt = xbase + k0;
-            const float *wt = LAYOUT == MAM_W_MK ? wbase + k0 : wbase + (int64_t)k0 * p.ldw;
-            float4 xr[(BN * KT / 4) / NT], wr[(BM * KT / 4) / NT];
-#pragma unroll
-            for (int it = 0; it < (BN * KT / 4) / NT; ++it)
-                xr[it] = *reinterpret_cast<const float4 *>(xt + xo[it]);
-#pragma unroll
-            for (int it = 0; it < (BM * KT / 4) / NT; ++it)
-                wr[it] = *reinterpret_cast<const float4 *>(wt + wo[it]);
-#pragma unroll
-            for (int it = 0; it < (BN * KT / 4) / NT; ++it) {
-                const int e = tid + it * NT;
-                *reinterpret_cast<float4 *>(&xs[e >> 3][(e & 7) * 4]) = xr[it];
-            }
-#pragma unroll
-            for (int it = 0; it < (BM * KT / 4) / NT; ++it) {
-                const int e = tid + it * NT;
-                if (LAYOUT == MAM_W_MK) {
-                    *reinterpret_cast<float4 *>(&ws[e >> 3][(e & 7) * 4]) = wr[it];
-                } else {
-                    const int c4 = (e & 7) + ((e >> 8) << 3);
-                    const int kk = (e >> 3) & 31;
-                    ws[c4 * 4 + 0][kk] = wr[it].x;
-                    ws[c4 * 4 + 1][kk] = wr[it].y;
-                    ws[c4 * 4 + 2][kk] = wr[it].z;
-                    ws[c4 * 4 + 3][kk] = wr[it].w;
-                }
+            if (LAYOUT == MAM_W_MK) {
+                dma_tile(xbase + k0, wbase + k0, dst, wave, doff, false);
+            } else {
+                // x by direct-to-LDS, w through registers
+                dma_tile(xbase + k0, xbase + k0, dst, wave, doff, true);
+                stage_w_km_fast(wbase + (int64_t)k0 * p.ldw, ws, tid, wo);
             }
         } else {
             stage_tile_generic<LAYOUT>(p, xs, ws, tid, row0, col0, k0, ke);
         }
-        __syncthreads();
+    };
 
-        // ---- 2 groups of 16 k: 32 outputs x 16 products each.  The two groups are unrolled
-        // so that the running extremes ping-pong between two register sets: the value before
-        // the group stays readable for the "did it improve" test without a copy. ----
-#pragma unroll
-        for (int gg = 0; gg < KT / G; ++gg) {
-            const uint32_t grel = (uint32_t)((k0 - kb) / G + gg);
-            float xv[TI][G];
-#pragma unroll
-            for (int i = 0; i < TI; ++i)
-#pragma unroll
-                for (int q = 0; q < G / 4; ++q) {
-                    const float4 t = *reinterpret_cast<const float4 *>(&xs[ty + 16 * i][gg * G + q * 4]);
-                    xv[i][q * 4 + 0] = t.x; xv[i][q * 4 + 1] = t.y;
-                    xv[i][q * 4 + 2] = t.z; xv[i][q * 4 + 3] = t.w;
-                }
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) {
-                float wv[G];
-#pragma unroll
-                for (int q = 0; q < G / 4; ++q) {
-                    const float4 t = *reinterpret_cast<const float4 *>(&ws[tx + 16 * j][gg * G + q * 4]);
-                    wv[q * 4 + 0] = t.x; wv[q * 4 + 1] = t.y;
-                    wv[q * 4 + 2] = t.z; wv[q * 4 + 3] = t.w;
-                }
-#pragma unroll
-                for (int i = 0; i < TI; ++i) {
-                    const float om = vmax[i][j], on = vmin[i][j];
-                    float hi = om, lo = on;
-#pragma unroll
-                    for (int q = 0; q < G; q += 2) {
-                        const float a = xv[i][q] * wv[q], b = xv[i][q + 1] * wv[q + 1];
-                        hi = __builtin_fmaxf(__builtin_fmaxf(hi, a), b);   // v_max3_f32
-                        lo = __builtin_fminf(__builtin_fminf(lo, a), b);   // v_min3_f32
-                    }
-                    if (ARGS) {
-                        // gsel.lo16 = (hi > om) ? grel : gsel.lo16 ; gsel.hi16 likewise for the min.
-                        // One compare and one sub-dword conditional move per extreme: the select
-                        // picks a 16-bit word of each source and writes one word of gsel.
-                        asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
-                            "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE "
-                            "src0_sel:WORD_0 src1_sel:WORD_0"
-                            : "+v"(gsel[i][j]) : "v"(hi), "v"(om), "v"(grel) : "vcc");
-                        asm("v_cmp_lt_f32 vcc, %1, %2\n\t"
-                            "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE "
-                            "src0_sel:WORD_1 src1_sel:WORD_0"
-                            : "+v"(gsel[i][j]) : "v"(lo), "v"(on), "v"(grel) : "vcc");
-                    }
-                    vmax[i][j] = hi;
-                    vmin[i][j] = lo;
-                }
-            }
-        }
+    stage(tile_a, 0);
+    __syncthreads();
+    for (int t = 0; t < ntiles; t += 2) {
+        // tile t from buffer A while tile t+1 lands in buffer B
+        if (t + 1 < ntiles) stage(tile_b, t + 1);
+        compute_tile<ARGS>(tile_a, tx, ty, (uint32_t)(t * (KT / G)), vmax, vmin, gsel);
+        __syncthreads();
+        if (t + 1 >= ntiles) break;
+        if (t + 2 < ntiles) stage(tile_a, t + 2);
+        compute_tile<ARGS>(tile_b, tx, ty, (uint32_t)((t + 1) * (KT / G)), vmax, vmin, gsel);
         __syncthreads();
     }
 
@@ -364,8 +430,8 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
         // of its results in its own LDS slots so that the index resolution can be a rolled loop
         // over j: one copy of the code per row instead of 32, and no register array indexed at
         // run time.
-        static_assert(3 * TJ * NT <= (BN + BM) * LDK, "result stash does not fit the tile buffer");
-        float *stash = smem + tid;
+        static_assert(3 * TJ * NT <= TILE_FLOATS, "result stash does not fit a tile buffer");
+        float *stash = tile_a + tid;
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
 #pragma unroll

@@ -28,7 +28,7 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
                                                     const int32_t *__restrict__ argmin,
                                                     int32_t *__restrict__ max_count,
                                                     int32_t *__restrict__ min_count, int N, int M,
-                                                    int K, int log2r, int kc, int vec)
+                                                    int K, int log2r, int kc, int vec, int vec_in)
 {
     extern __shared__ uint32_t cnt[];  // [R][kc]
     const int tid = threadIdx.x;
@@ -41,14 +41,32 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
         const int nn = (N - n0) < ROWS_PER_PASS ? (N - n0) : ROWS_PER_PASS;
         for (int i = tid; i < R * kc; i += NT_H) cnt[i] = 0u;
         __syncthreads();
-        const int pairs = nn << log2r;
-        for (int pi = tid; pi < pairs; pi += NT_H) {
-            const int n = n0 + (pi >> log2r), r = pi & (R - 1);
-            if (r >= rn) continue;
-            const int64_t o = (int64_t)n * M + m0 + r;
-            const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
-            if ((unsigned)a1 < (unsigned)kn) atomicAdd(&cnt[r * kc + a1], 1u);
-            if ((unsigned)a2 < (unsigned)kn) atomicAdd(&cnt[r * kc + a2], 0x10000u);
+        if (vec_in && rn == R) {
+            const int qpr = R >> 2;
+            const int items = nn * qpr;
+            for (int it = tid; it < items; it += NT_H) {
+                const int n = n0 + it / qpr, r0 = (it % qpr) * 4;
+                const int64_t o = (int64_t)n * M + m0 + r0;
+                const int4 i1 = *reinterpret_cast<const int4 *>(argmax + o);
+                const int4 i2 = *reinterpret_cast<const int4 *>(argmin + o);
+                const int a1[4] = {i1.x - k0, i1.y - k0, i1.z - k0, i1.w - k0};
+                const int a2[4] = {i2.x - k0, i2.y - k0, i2.z - k0, i2.w - k0};
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if ((unsigned)a1[u] < (unsigned)kn) atomicAdd(&cnt[(r0 + u) * kc + a1[u]], 1u);
+                    if ((unsigned)a2[u] < (unsigned)kn) atomicAdd(&cnt[(r0 + u) * kc + a2[u]], 0x10000u);
+                }
+            }
+        } else {
+            const int pairs = nn << log2r;
+            for (int pi = tid; pi < pairs; pi += NT_H) {
+                const int n = n0 + (pi >> log2r), r = pi & (R - 1);
+                if (r >= rn) continue;
+                const int64_t o = (int64_t)n * M + m0 + r;
+                const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
+                if ((unsigned)a1 < (unsigned)kn) atomicAdd(&cnt[r * kc + a1], 1u);
+                if ((unsigned)a2 < (unsigned)kn) atomicAdd(&cnt[r * kc + a2], 0x10000u);
+            }
         }
         __syncthreads();
         // Stream the slab back: 4 cells per lane, whole 16-byte chunks skipped when nothing in
@@ -56,22 +74,41 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
         // a coalesced read-modify-write of the slab; at small N*M it degenerates to a sparse one.
         if (vec) {
             const int q = kn >> 2;
-            for (int e = tid; e < rn * q; e += NT_H) {
-                const int r = e / q, c4 = e - r * q;
-                const uint4 v = *reinterpret_cast<const uint4 *>(&cnt[r * kc + c4 * 4]);
-                if ((v.x | v.y | v.z | v.w) == 0u) continue;
-                const int64_t cell = (int64_t)(m0 + r) * K + k0 + c4 * 4;
-                if ((v.x | v.y | v.z | v.w) & 0xffffu) {
-                    int4 a = *reinterpret_cast<int4 *>(max_count + cell);
-                    a.x += (int)(v.x & 0xffffu); a.y += (int)(v.y & 0xffffu);
-                    a.z += (int)(v.z & 0xffffu); a.w += (int)(v.w & 0xffffu);
-                    *reinterpret_cast<int4 *>(max_count + cell) = a;
+            const int total = rn * q;
+            for (int eb = tid; eb < total; eb += 4 * NT_H) {
+                uint4 v[4];
+                int4 amx[4], amn[4];
+                int64_t cell[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int e = eb + u * NT_H;
+                    v[u] = make_uint4(0u, 0u, 0u, 0u);
+                    cell[u] = 0;
+                    if (e < total) {
+                        const int r = e / q, c4 = e - r * q;
+                        v[u] = *reinterpret_cast<const uint4 *>(&cnt[r * kc + c4 * 4]);
+                        cell[u] = (int64_t)(m0 + r) * K + k0 + c4 * 4;
+                    }
                 }
-                if ((v.x | v.y | v.z | v.w) >> 16) {
-                    int4 a = *reinterpret_cast<int4 *>(min_count + cell);
-                    a.x += (int)(v.x >> 16); a.y += (int)(v.y >> 16);
-                    a.z += (int)(v.z >> 16); a.w += (int)(v.w >> 16);
-                    *reinterpret_cast<int4 *>(min_count + cell) = a;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t any = v[u].x | v[u].y | v[u].z | v[u].w;
+                    if (any & 0xffffu) amx[u] = *reinterpret_cast<const int4 *>(max_count + cell[u]);
+                    if (any >> 16) amn[u] = *reinterpret_cast<const int4 *>(min_count + cell[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint32_t any = v[u].x | v[u].y | v[u].z | v[u].w;
+                    if (any & 0xffffu) {
+                        amx[u].x += (int)(v[u].x & 0xffffu); amx[u].y += (int)(v[u].y & 0xffffu);
+                        amx[u].z += (int)(v[u].z & 0xffffu); amx[u].w += (int)(v[u].w & 0xffffu);
+                        *reinterpret_cast<int4 *>(max_count + cell[u]) = amx[u];
+                    }
+                    if (any >> 16) {
+                        amn[u].x += (int)(v[u].x >> 16); amn[u].y += (int)(v[u].y >> 16);
+                        amn[u].z += (int)(v[u].z >> 16); amn[u].w += (int)(v[u].w >> 16);
+                        *reinterpret_cast<int4 *>(min_count + cell[u]) = amn[u];
+                    }
                 }
             }
         } else {
@@ -125,15 +162,6 @@ __global__ __launch_bounds__(NT) void reference_kernel(const int32_t *__restrict
     }
 }
 
-static int lds_budget_words(const void *kernel)
-{
-    constexpr int kWant = 128 * 1024;
-    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kWant) == hipSuccess)
-        return kWant / 4;
-    (void)hipGetLastError();
-    return 64 * 1024 / 4;
-}
-
 }  // namespace selcount
 }  // namespace mam
 
@@ -152,17 +180,19 @@ extern "C" int mam_selection_count(const int32_t *argmax, const int32_t *argmin,
         return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (mode == MAM_COUNT_HITS) {
-        static const int budget = selcount::lds_budget_words((const void *)selcount::hits_kernel);
-        const int log2r = 3;
+        // 4 whole-K rows of packed counters in 64 KiB: two workgroups per CU
+        const int budget = 64 * 1024 / 4;
+        const int log2r = 2;
         const int R = 1 << log2r;
         int kc = budget / R;
         if (K < kc) kc = (int)((K + 3) / 4 * 4);
         const int64_t ktiles = ceil_div(K, kc);
         const int vec = (K % 4 == 0) && ((uintptr_t)max_count % 16 == 0) && ((uintptr_t)min_count % 16 == 0);
+        const int vec_in = (M % 4 == 0) && ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0);
         if (ktiles > 65535) return fail(MAM_ERR_UNSUPPORTED, "K too large for the selection-count grid");
         hipLaunchKernelGGL(selcount::hits_kernel, dim3((unsigned)ceil_div(M, R), (unsigned)ktiles),
                            dim3(selcount::NT_H), (size_t)R * kc * 4, st, argmax, argmin, max_count,
-                           min_count, (int)N, (int)M, (int)K, log2r, kc, vec);
+                           min_count, (int)N, (int)M, (int)K, log2r, kc, vec, vec_in);
         return check_launch("selcount::hits_kernel");
     }
     const int words = (int)ceil_div(K, 32);
