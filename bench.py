@@ -96,19 +96,20 @@ def main():
     min_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
     ws_bytes = lib.mam_fc_forward_workspace(N, K, M)
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    wsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)   # selected weights, forward -> backward
 
     stream = torch.cuda.current_stream(dev)
     sp = ctypes.c_void_p(stream.cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
 
     def forward():
-        rc = lib.mam_fc_forward(P(x), K, P(w), K, capi.W_MK, None, P(c), P(amax), P(amin), N, K, M,
-                                P(ws), ws_bytes, sp)
+        rc = lib.mam_fc_forward(P(x), K, P(w), K, capi.W_MK, None, P(c), P(amax), P(amin), P(wsel),
+                                N, K, M, P(ws), ws_bytes, sp)
         assert rc == 0, lib.mam_last_error()
 
     def backward():
-        rc = lib.mam_fc_backward(P(x), K, P(w), K, capi.W_MK, P(g), P(amax), P(amin), P(xg), P(wg),
-                                 N, K, M, sp)
+        rc = lib.mam_fc_backward(P(x), K, P(w), K, capi.W_MK, P(g), P(amax), P(amin), P(wsel), P(xg),
+                                 P(wg), N, K, M, sp)
         assert rc == 0, lib.mam_last_error()
 
     def count():

@@ -42,12 +42,12 @@ def lib():
             fn = getattr(l, name)
             fn.restype = _size
             fn.argtypes = [_i64, _i64, _i64]
-        l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64,
-                                     _ptr, _size, _ptr]
+        l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
+                                     _i64, _ptr, _size, _ptr]
         l.mam_fc_forward_values.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _i64, _i64, _i64,
                                             _ptr, _size, _ptr]
-        l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
-                                      _i64, _ptr]
+        l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
+                                      _i64, _i64, _ptr]
         l.mam_selection_count.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr]
         l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
                                          _i64, _ptr, _size, _ptr]
@@ -87,8 +87,9 @@ def _ld(t):
     return t.stride(0) if t.size(0) > 1 else max(t.size(1), 1)
 
 
-def fc_forward(x, w, layout=W_KM, bias=None, workspace=None):
-    """-> (c, argmax, argmin) on x.device.  ``workspace`` (uint8 tensor) is allocated if None."""
+def fc_forward(x, w, layout=W_KM, bias=None, workspace=None, w_sel=None):
+    """-> (c, argmax, argmin) on x.device.  ``workspace`` (uint8 tensor) is allocated if None.
+    ``w_sel``: optional (2, N, M) fp32 tensor that receives the selected weights."""
     l = lib()
     N, K, M = _dims(x, w, layout)
     c = torch.empty((N, M), dtype=torch.float32, device=x.device)
@@ -99,7 +100,7 @@ def fc_forward(x, w, layout=W_KM, bias=None, workspace=None):
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         _check(l.mam_fc_forward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(bias), _p(c), _p(amax), _p(amin),
-                                N, K, M, _p(workspace), 0 if workspace is None else workspace.numel(),
+                                _p(w_sel), N, K, M, _p(workspace), 0 if workspace is None else workspace.numel(),
                                 _stream(x)))
     return c, amax, amin
 
@@ -118,7 +119,7 @@ def fc_forward_values(x, w, layout=W_KM, bias=None, workspace=None):
     return c
 
 
-def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=True):
+def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=True, w_sel=None):
     """-> (x_grad or None, w_grad or None); w_grad has the shape and layout of w."""
     l = lib()
     N, K, M = _dims(x, w, layout)
@@ -126,7 +127,7 @@ def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=Tru
     wg = torch.empty(tuple(w.shape), dtype=torch.float32, device=x.device) if want_w else None
     with torch.cuda.device(x.device):
         _check(l.mam_fc_backward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(grad), _p(argmax), _p(argmin),
-                                 _p(xg), _p(wg), N, K, M, _stream(x)))
+                                 _p(w_sel), _p(xg), _p(wg), N, K, M, _stream(x)))
     return xg, wg
 
 

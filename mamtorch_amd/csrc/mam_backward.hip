@@ -33,7 +33,7 @@ template <int LAYOUT>
 __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
     const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    float *__restrict__ x_grad, int K, int M, int kc)
+    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int K, int M, int kc)
 {
     extern __shared__ float hist[];
     const int n = blockIdx.x;
@@ -61,8 +61,15 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int m = mb + u * NT_X;
-                wv1[u] = (unsigned)a1[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a1[u] + k0, m) : 0.0f;
-                wv2[u] = (unsigned)a2[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a2[u] + k0, m) : 0.0f;
+                // the forward can hand over the selected weights; otherwise gather them
+                if (w_sel) {
+                    const bool ok = m < M;
+                    wv1[u] = ok ? w_sel[(int64_t)n * M + m] : 0.0f;
+                    wv2[u] = ok ? w_sel[nm + (int64_t)n * M + m] : 0.0f;
+                } else {
+                    wv1[u] = (unsigned)a1[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a1[u] + k0, m) : 0.0f;
+                    wv2[u] = (unsigned)a2[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a2[u] + k0, m) : 0.0f;
+                }
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
@@ -180,16 +187,16 @@ static int lds_budget_floats(const void *kernel)
 
 template <int LAYOUT>
 static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ldw, const float *grad,
-                         const int32_t *argmax, const int32_t *argmin, float *x_grad, float *w_grad,
-                         int64_t N, int64_t K, int64_t M, hipStream_t st)
+                         const int32_t *argmax, const int32_t *argmin, const float *w_sel,
+                         float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
 {
     int rc = MAM_OK;
     if (x_grad) {
         static const int budget = lds_budget_floats((const void *)mam_bwd_x_kernel<LAYOUT>);
         const int kc = (int)(K < budget ? K : budget);
         hipLaunchKernelGGL((mam_bwd_x_kernel<LAYOUT>), dim3((unsigned)N), dim3(NT_X),
-                           (size_t)kc * sizeof(float), st, w, ldw, grad, argmax, argmin, x_grad,
-                           (int)K, (int)M, kc);
+                           (size_t)kc * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M,
+                           x_grad, (int)K, (int)M, kc);
         rc = check_launch("mam_bwd_x_kernel");
         if (rc != MAM_OK) return rc;
     }
@@ -220,8 +227,8 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
 
 extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                                const float *grad, const int32_t *argmax, const int32_t *argmin,
-                               float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M,
-                               void *stream)
+                               const float *w_sel, float *x_grad, float *w_grad, int64_t N, int64_t K,
+                               int64_t M, void *stream)
 {
     using namespace mam;
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
@@ -241,6 +248,6 @@ extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int6
     if (ldx < K || ldw < (w_layout == MAM_W_MK ? K : M))
         return fail(MAM_ERR_INVALID_ARGUMENT, "leading dimension smaller than the row length");
     if (w_layout == MAM_W_MK)
-        return bwd::launch_layout<MAM_W_MK>(x, ldx, w, ldw, grad, argmax, argmin, x_grad, w_grad, N, K, M, st);
-    return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, x_grad, w_grad, N, K, M, st);
+        return bwd::launch_layout<MAM_W_MK>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_grad, w_grad, N, K, M, st);
+    return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_grad, w_grad, N, K, M, st);
 }

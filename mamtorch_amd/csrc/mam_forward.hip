@@ -58,11 +58,13 @@ struct Params {
     float *c;
     int32_t *argmax;
     int32_t *argmin;
+    float *wsel;      // optional [2][N*M]: the selected weights w[argmax], w[argmin] (for the backward)
     float *part;      // split-K partials: [split][3 or 2][N*M]: max, min, (group ids packed 16:16)
     int N, K, M;
     int tiles_n, tiles_m, splits, k_per_split;
     int vec_x, vec_w;  // 16-byte global loads are legal for x / w
     int fast;          // the k-invariant 32-bit-offset staging path is legal
+    int coop;          // the cooperative resolve is legal: (M,K) w, 16-byte rows, K % G == 0
 };
 
 // First k in group g (ascending) whose product equals `target`; value recomputed from it.
@@ -70,13 +72,14 @@ struct Params {
 // G operands of each side are fetched with 16-byte loads when the layout allows it.
 template <int LAYOUT>
 __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, float target,
-                                        float &val, int &idx)
+                                        float &val, int &idx, float &wsel)
 {
     const int kb = g * G;
     const int klast = p.K - 1;
     idx = kb < klast ? kb : klast;
     val = target;
     const float *xr = p.x + (int64_t)n * p.ldx;
+    wsel = load_w<LAYOUT>(p.w, p.ldw, idx, m);
     float xv[G], wv[G];
     const bool whole = kb + G <= p.K;
     if (whole && p.vec_x) {
@@ -104,7 +107,7 @@ __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, fl
 #pragma unroll
     for (int kk = G - 1; kk >= 0; --kk) {
         const float prod = xv[kk] * wv[kk];
-        if (prod == target) { idx = (kb + kk) < klast ? (kb + kk) : klast; val = prod; }
+        if (prod == target) { idx = (kb + kk) < klast ? (kb + kk) : klast; val = prod; wsel = wv[kk]; }
     }
 }
 
@@ -128,9 +131,10 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
 {
     float hi = vmax, lo = vmin;
     int ih = 0, il = 0;
+    float wh = 0.0f, wl = 0.0f;
     if (ARGS) {
-        resolve<LAYOUT>(p, n, m, gmax, vmax, hi, ih);
-        resolve<LAYOUT>(p, n, m, gmin, vmin, lo, il);
+        resolve<LAYOUT>(p, n, m, gmax, vmax, hi, ih, wh);
+        resolve<LAYOUT>(p, n, m, gmin, vmin, lo, il, wl);
     } else {
         if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m);
         if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m);
@@ -142,6 +146,77 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
     if (ARGS) {
         p.argmax[o] = ih;
         p.argmin[o] = il;
+        if (p.wsel) {
+            p.wsel[o] = wh;
+            p.wsel[(int64_t)p.N * p.M + o] = wl;
+        }
+    }
+}
+
+// Cooperative resolve of the 64 outputs held by one wave (fast layouts only: (M,K) weight,
+// 16-byte aligned rows, K a multiple of G).  The cost of resolving is cache-line lookups, so the
+// G/4 lanes of a task each fetch one 16-byte chunk of x and of w: a task touches one contiguous
+// G*4-byte segment per operand instead of G/4 lanes each touching G/4 segments.  128 tasks
+// (64 outputs x {max, min}) are processed 64/(G/4) per round.
+//   vals : LDS, [2][64]  running max, running min of the wave's outputs
+//   grps : LDS, [2][64]  absolute group id of the max, of the min
+//   nm_of(slot, n, m, valid): output coordinates of slot 0..63 (clamped into range when !valid)
+constexpr int LPT = G / 4;             // lanes per task
+constexpr int TPR = 64 / LPT;          // tasks per round
+constexpr int RES_ROUNDS = 128 / TPR;
+
+template <class NM>
+__device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps,
+                                             int lane, NM nm_of)
+{
+    // rounds are unrolled so that the loads of all of them are in flight together
+#pragma unroll
+    for (int r = 0; r < RES_ROUNDS; ++r) {
+        const int task = r * TPR + lane / LPT;
+        const int slot = task >> 1, ext = task & 1, sub = lane % LPT;
+        int n, m;
+        bool valid;
+        nm_of(slot, n, m, valid);
+        const float target = vals[ext * 64 + slot];
+        const int g = grps[ext * 64 + slot];
+        const int kb = g * G + sub * 4;
+        const float4 xa = *reinterpret_cast<const float4 *>(p.x + (int64_t)n * p.ldx + kb);
+        const float4 wa = *reinterpret_cast<const float4 *>(p.w + (int64_t)m * p.ldw + kb);
+        const float p0 = xa.x * wa.x, p1 = xa.y * wa.y, p2 = xa.z * wa.z, p3 = xa.w * wa.w;
+        // position within the group of this lane's first match (lowest wins), 255 = none
+        int key = 255;
+        float val = target;
+        float wsel = wa.x;         // fallback: the first weight of the group (only lane sub 0 can keep it)
+        if (p3 == target) { key = sub * 4 + 3; val = p3; wsel = wa.w; }
+        if (p2 == target) { key = sub * 4 + 2; val = p2; wsel = wa.z; }
+        if (p1 == target) { key = sub * 4 + 1; val = p1; wsel = wa.y; }
+        if (p0 == target) { key = sub * 4 + 0; val = p0; wsel = wa.x; }
+        if (key == 255 && sub == 0) key = 254;   // no match anywhere: lane 0's fallback wins the reduce
+#pragma unroll
+        for (int off = 1; off < LPT; off <<= 1) {
+            const int okey = __shfl_xor(key, off);
+            const float oval = __shfl_xor(val, off);
+            const float owsel = __shfl_xor(wsel, off);
+            if (okey < key) { key = okey; val = oval; wsel = owsel; }
+        }
+        if (key >= 254) key = 0;   // no product equals the extreme (NaN operands): first of the group
+        const int idx = g * G + key;
+        // lanes of the max task and of the min task of one output are LPT apart
+        const float val_min = __shfl_xor(val, LPT);
+        const int idx_min = __shfl_xor(idx, LPT);
+        const float wsel_min = __shfl_xor(wsel, LPT);
+        if (ext == 0 && sub == 0 && valid) {
+            float sum = val + val_min;
+            if (p.bias) sum = sum + p.bias[m];
+            const int64_t o = (int64_t)n * p.M + m;
+            p.c[o] = sum;
+            p.argmax[o] = idx;
+            p.argmin[o] = idx_min;
+            if (p.wsel) {
+                p.wsel[o] = wsel;
+                p.wsel[(int64_t)p.N * p.M + o] = wsel_min;
+            }
+        }
     }
 }
 
@@ -425,11 +500,41 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 
     // ---- epilogue ----
     const int g0 = kb / G;
-    if (p.splits == 1) {
-        // The tiles in LDS are dead (the k loop ended on a barrier).  Each thread parks one row
-        // of its results in its own LDS slots so that the index resolution can be a rolled loop
-        // over j: one copy of the code per row instead of 32, and no register array indexed at
-        // run time.
+    if (p.splits == 1 && ARGS && p.coop) {
+        // The tiles in LDS are dead (the k loop ended on a barrier).  Row by row, each wave parks
+        // its 64 x 8 results in LDS and resolves them cooperatively.
+        static_assert(2 * TJ * NT <= TILE_FLOATS, "result stash does not fit a tile buffer");
+        const int lane = tid & 63;
+        float *vals = tile_a + wave * (TJ * 2 * 64);
+        int *grps = reinterpret_cast<int *>(tile_b) + wave * (TJ * 2 * 64);
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                vals[(j * 2 + 0) * 64 + lane] = vmax[i][j];
+                vals[(j * 2 + 1) * 64 + lane] = vmin[i][j];
+                grps[(j * 2 + 0) * 64 + lane] = g0 + (int)(gsel[i][j] & 0xffffu);
+                grps[(j * 2 + 1) * 64 + lane] = g0 + (int)(gsel[i][j] >> 16);
+            }
+            __syncthreads();
+#pragma unroll 1
+            for (int j = 0; j < TJ; ++j) {
+                const int nbase = row0 + 16 * i + 4 * wave, mbase = col0 + 16 * j;
+                resolve_wave(p, vals + j * 128, grps + j * 128, lane,
+                             [&](int slot, int &n, int &m, bool &valid) {
+                                 n = nbase + (slot >> 4);
+                                 m = mbase + (slot & 15);
+                                 valid = n < p.N && m < p.M;
+                                 n = n < p.N ? n : p.N - 1;
+                                 m = m < p.M ? m : p.M - 1;
+                             });
+            }
+        }
+    } else if (p.splits == 1) {
+        // Generic layouts: each thread parks one row of its results in its own LDS slots so that
+        // the index resolution can be a rolled loop over j (one copy of the code per row, and no
+        // register array indexed at run time).
         static_assert(3 * TJ * NT <= TILE_FLOATS, "result stash does not fit a tile buffer");
         float *stash = tile_a + tid;
 #pragma unroll
@@ -476,34 +581,66 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 template <int LAYOUT, bool ARGS>
 __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
 {
+    // A workgroup owns a 16 x 16 patch of c.  Resolving re-reads G weights of row m per output,
+    // i.e. random lines of the weight matrix; ordering the patches so that all batch patches of
+    // one 16-neuron range run back to back on one XCD keeps those 16 weight rows in that L2.
+    __shared__ float vals_s[4][2][64];
+    __shared__ int grps_s[4][2][64];
     const int64_t nm = (int64_t)p.N * p.M;
-    const int64_t o = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (o >= nm) return;
+    const int patches_n = (p.N + 15) / 16;
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int pm = logical / patches_n, pn = logical - pm * patches_n;
+    const int n_own = pn * 16 + (threadIdx.x >> 4), m_own = pm * 16 + (threadIdx.x & 15);
+    const bool live = n_own < p.N && m_own < p.M;
+    const int64_t o = (int64_t)n_own * p.M + m_own;
     const int stride = ARGS ? 3 : 2;
     const int gps = p.k_per_split / G;   // groups per split
-    float vmax = p.part[o], vmin = p.part[nm + o];
+    float vmax = 0.0f, vmin = 0.0f;
     int gmax = 0, gmin = 0;
-    if (ARGS) {
-        const int pk = __float_as_int(p.part[2 * nm + o]);
-        gmax = pk & 0xffff;
-        gmin = (pk >> 16) & 0xffff;
-    }
-    for (int s = 1; s < p.splits; ++s) {
-        const float *base = p.part + (int64_t)s * stride * nm;
-        const float hi = base[o], lo = base[nm + o];
-        int pk = 0;
-        if (ARGS) pk = __float_as_int(base[2 * nm + o]);
-        if (hi > vmax) {
-            vmax = hi;
-            gmax = s * gps + (pk & 0xffff);
+    if (live) {
+        vmax = p.part[o];
+        vmin = p.part[nm + o];
+        if (ARGS) {
+            const int pk = __float_as_int(p.part[2 * nm + o]);
+            gmax = pk & 0xffff;
+            gmin = (pk >> 16) & 0xffff;
         }
-        if (lo < vmin) {
-            vmin = lo;
-            gmin = s * gps + ((pk >> 16) & 0xffff);
+        for (int s = 1; s < p.splits; ++s) {
+            const float *base = p.part + (int64_t)s * stride * nm;
+            const float hi = base[o], lo = base[nm + o];
+            int pk = 0;
+            if (ARGS) pk = __float_as_int(base[2 * nm + o]);
+            if (hi > vmax) {
+                vmax = hi;
+                gmax = s * gps + (pk & 0xffff);
+            }
+            if (lo < vmin) {
+                vmin = lo;
+                gmin = s * gps + ((pk >> 16) & 0xffff);
+            }
         }
     }
-    const int n = (int)(o / p.M), m = (int)(o - (int64_t)n * p.M);
-    finish<LAYOUT, ARGS>(p, n, m, vmax, vmin, gmax, gmin);
+    if (ARGS && p.coop) {
+        const int lane = threadIdx.x & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        vals_s[wave][0][lane] = vmax;
+        vals_s[wave][1][lane] = vmin;
+        grps_s[wave][0][lane] = gmax;
+        grps_s[wave][1][lane] = gmin;
+        __syncthreads();
+        const int nbase = pn * 16 + 4 * wave, mbase = pm * 16;
+        resolve_wave(p, &vals_s[wave][0][0], &grps_s[wave][0][0], lane,
+                     [&](int slot, int &n, int &m, bool &valid) {
+                         n = nbase + (slot >> 4);
+                         m = mbase + (slot & 15);
+                         valid = n < p.N && m < p.M;
+                         n = n < p.N ? n : p.N - 1;
+                         m = m < p.M ? m : p.M - 1;
+                     });
+        return;
+    }
+    if (!live) return;
+    finish<LAYOUT, ARGS>(p, n_own, m_own, vmax, vmin, gmax, gmin);
 }
 
 // How many K ranges to split into so that at least two workgroups reach every CU.
@@ -531,7 +668,7 @@ static size_t workspace_bytes(int64_t N, int64_t K, int64_t M, bool args)
 
 template <bool ARGS>
 static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
-                  const float *bias, float *c, int32_t *argmax, int32_t *argmin, int64_t N,
+                  const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, int64_t N,
                   int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream)
 {
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
@@ -548,7 +685,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
 
     Params p;
     p.x = x; p.ldx = ldx; p.w = w; p.ldw = ldw; p.bias = bias;
-    p.c = c; p.argmax = argmax; p.argmin = argmin;
+    p.c = c; p.argmax = argmax; p.argmin = argmin; p.wsel = w_sel;
     p.N = (int)N; p.K = (int)K; p.M = (int)M;
     p.tiles_n = (int)ceil_div(N, BN);
     p.tiles_m = (int)ceil_div(M, BM);
@@ -568,6 +705,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     // the fast staging path addresses a tile with 32-bit element offsets from the tile base
     const int64_t w_rows = (w_layout == MAM_W_MK) ? fwd::BM : fwd::KT;
     p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30));
+    p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0);
     // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
     if ((int64_t)p.k_per_split / G > 65536)
         return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds %d per K range", (long long)K, 65536 * G);
@@ -582,7 +720,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     int rc = check_launch("mam_fwd_kernel");
     if (rc != MAM_OK) return rc;
     if (p.splits > 1) {
-        const unsigned mb = (unsigned)ceil_div(N * M, 256);
+        const unsigned mb = (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
         if (w_layout == MAM_W_MK)
             hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS>), dim3(mb), dim3(256), 0, st, p);
         else
@@ -609,10 +747,10 @@ extern "C" size_t mam_fc_forward_values_workspace(int64_t N, int64_t K, int64_t 
 
 extern "C" int mam_fc_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                               const float *bias, float *c, int32_t *argmax, int32_t *argmin,
-                              int64_t N, int64_t K, int64_t M, void *workspace,
+                              float *w_sel, int64_t N, int64_t K, int64_t M, void *workspace,
                               size_t workspace_bytes, void *stream)
 {
-    return mam::fwd::launch<true>(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, N, K, M,
+    return mam::fwd::launch<true>(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, N, K, M,
                                   workspace, workspace_bytes, stream);
 }
 
@@ -620,6 +758,6 @@ extern "C" int mam_fc_forward_values(const float *x, int64_t ldx, const float *w
                                      int w_layout, const float *bias, float *c, int64_t N, int64_t K,
                                      int64_t M, void *workspace, size_t workspace_bytes, void *stream)
 {
-    return mam::fwd::launch<false>(x, ldx, w, ldw, w_layout, bias, c, nullptr, nullptr, N, K, M,
+    return mam::fwd::launch<false>(x, ldx, w, ldw, w_layout, bias, c, nullptr, nullptr, nullptr, N, K, M,
                                    workspace, workspace_bytes, stream);
 }

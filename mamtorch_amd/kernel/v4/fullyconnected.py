@@ -6,7 +6,9 @@ served by the exact kernel, so its error against the oracle is zero.
 
 ``fullyconnected_wt`` is an addition: it takes the module's ``weight`` (out, in) as stored, so no
 transposed copy of the weight is made per call, adds the bias inside the kernel, and returns the
-weight gradient in (out, in) layout.
+weight gradient in (out, in) layout.  The raw operator returns a fourth tensor, the selected
+weights w[argmax] / w[argmin] of shape (2, N, out): the index resolution has them in hand, and
+the backward then needs no random reads of the weight matrix.
 """
 import torch
 from torch import Tensor
@@ -25,7 +27,7 @@ def fullyconnected(a: Tensor, b: Tensor) -> list[Tensor]:
 
 def fullyconnected_wt(a: Tensor, weight: Tensor, bias=None) -> list[Tensor]:
     """a (N, in), weight (out, in), bias (out) or None -> [C, argmax, argmin]."""
-    return K.fullyconnected_wt.default(a, weight, bias)
+    return K.fullyconnected_wt.default(a, weight, bias)[:3]
 
 
 register_exact_forward(library_name)
@@ -41,11 +43,12 @@ def _(a, weight, bias):
     shape = (a.size(0), weight.size(0))
     return [torch.empty(shape, dtype=torch.float, device=a.device),
             torch.empty(shape, dtype=torch.int, device=a.device),
-            torch.empty(shape, dtype=torch.int, device=a.device)]
+            torch.empty(shape, dtype=torch.int, device=a.device),
+            torch.empty((2,) + shape, dtype=torch.float, device=a.device)]
 
 
 @torch.library.register_fake(f"{library_name}::fullyconnected_wt_backward")
-def _(a, weight, grad, argmax, argmin):
+def _(a, weight, grad, argmax, argmin, w_sel):
     torch._check(a.size(1) == weight.size(1))
     torch._check(grad.size(0) == a.size(0))
     torch._check(grad.size(1) == weight.size(0))
@@ -59,17 +62,18 @@ def _(a, weight, grad, argmax, argmin):
 
 def _wt_setup_context(ctx, inputs, output):
     a, weight, bias = inputs
-    _, argmax, argmin = output
+    _, argmax, argmin, w_sel = output
     need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
-    ctx.save_for_backward(a if need else None, weight if need else None, argmax, argmin)
+    ctx.save_for_backward(a if need else None, weight if need else None, argmax, argmin,
+                          w_sel if need else None)
 
 
 def _wt_backward(ctx, grad):
-    a, weight, argmax, argmin = ctx.saved_tensors
+    a, weight, argmax, argmin, w_sel = ctx.saved_tensors
     a_grad, w_grad, bias_grad = None, None, None
     g = grad[0]
     if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-        a_grad, w_grad = K.fullyconnected_wt_backward.default(a, weight, g.contiguous(), argmax, argmin)
+        a_grad, w_grad = K.fullyconnected_wt_backward.default(a, weight, g.contiguous(), argmax, argmin, w_sel)
     if ctx.needs_input_grad[2]:
         bias_grad = g.sum(dim=0)
     return a_grad, w_grad, bias_grad

@@ -185,7 +185,7 @@ class FullyConnected(Module):
                                                w.narrow(1, self.in_features - last, last), None)
         else:
             if self.store_args:
-                C_flat, argmax, argmin = K.v4.fullyconnected_wt(input_flat, w, fused)
+                C_flat, argmax, argmin = K.v4.fullyconnected_wt(input_flat, w, fused)[:3]
                 self.argmax = argmax
                 self.argmin = argmin
             else:

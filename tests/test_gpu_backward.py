@@ -40,7 +40,12 @@ def _check(x, w_mk, grad, amax, amin, what, layouts=(0, 1)):
     for layout in layouts:
         wd = (w_mk if layout == capi.W_MK else w_mk.T).contiguous().to(dev)
         xg, wg = capi.fc_backward(xd, wd, gd, a1, a2, layout)
+        # the same call with the selected weights handed over instead of gathered
+        cols = torch.arange(w_mk.shape[0])[None, :]
+        w_sel = torch.stack([w_mk[cols, torch.tensor(amax).long()], w_mk[cols, torch.tensor(amin).long()]]).to(dev)
+        xg2, _ = capi.fc_backward(xd, wd, gd, a1, a2, layout, want_w=False, w_sel=w_sel.contiguous())
         torch.cuda.synchronize()
+        close(xg2.cpu().numpy(), xo, xs, "%s x_grad (w_sel) layout %d" % (what, layout))
         wg = wg.cpu().numpy() if layout == capi.W_MK else wg.cpu().numpy().T
         close(xg.cpu().numpy(), xo, xs, "%s x_grad layout %d" % (what, layout))
         close(wg, wo, ws_, "%s w_grad layout %d" % (what, layout))

@@ -267,3 +267,22 @@ def test_large_batch_inference_config4(M):
     # the (K, M) operand gives the same answer
     c2, amax2, amin2 = capi.fc_forward(xd[:2048], wd.T.contiguous(), capi.W_KM)
     assert torch.equal(c2, c[:2048]) and torch.equal(amax2, amax[:2048]) and torch.equal(amin2, amin[:2048])
+
+
+@pytest.mark.parametrize("shape", [(64, 784, 256), (256, 4096, 512), (70, 123, 45), (300, 2048, 200)])
+def test_selected_weights_output(shape):
+    """w_sel[0] = w[argmax[n,m], m], w_sel[1] = w[argmin[n,m], m] (exact copies), both layouts."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    N, K, M = shape
+    x, w, _ = random_case(N, K, M, seed=11)
+    want = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+    cols = np.arange(M)[None, :]
+    for layout, wl in ((capi.W_MK, w.contiguous()), (capi.W_KM, w.T.contiguous())):
+        w_sel = torch.full((2, N, M), float("nan"), device=dev)
+        c, amax, amin = capi.fc_forward(x.to(dev), wl.to(dev), layout, w_sel=w_sel)
+        torch.cuda.synchronize()
+        assert_index_equal(amax.cpu().numpy(), want[1], "argmax")
+        assert_bits_equal(w_sel[0].cpu().numpy(), w.numpy()[cols, want[1]], "w_sel max layout %d" % layout)
+        assert_bits_equal(w_sel[1].cpu().numpy(), w.numpy()[cols, want[2]], "w_sel min layout %d" % layout)
