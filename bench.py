@@ -117,6 +117,11 @@ def main():
                                      capi.COUNT_HITS, sp)
         assert rc == 0, lib.mam_last_error()
 
+    # one plain 64 MiB copy kernel: the known-size reference that scales the profiler's
+    # FETCH_SIZE / WRITE_SIZE counters when traffic is measured
+    calibration_copy = max_count.clone()
+    del calibration_copy
+
     for _ in range(args.warmup):
         forward(); backward(); count()
     torch.cuda.synchronize()

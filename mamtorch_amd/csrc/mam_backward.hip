@@ -84,74 +84,44 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
     }
 }
 
+// Scatter of one (batch row, 4 consecutive neurons) item into the slab histogram.
 template <int LAYOUT>
-__global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
-    const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
-    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    float *__restrict__ w_grad, int N, int K, int M, int log2r, int kc, int vec_out,
-    int vec_in)
+__device__ __forceinline__ void scatter_quad(float *hist, const float4 &g, const int4 &i1, const int4 &i2,
+                                             const float (&x1)[4], const float (&x2)[4], int r0, int k0,
+                                             int kn, int kc, int log2r)
 {
-    extern __shared__ float hist[];
-    const int tid = threadIdx.x;
-    const int R = 1 << log2r;
-    const int mt = xcd_remap(blockIdx.x, gridDim.x);
-    const int m0 = mt * R;
-    const int k0 = blockIdx.y * kc;
-    const int rn = (M - m0) < R ? (M - m0) : R;
-    const int kn = (K - k0) < kc ? (K - k0) : kc;
-
-    const int cells = R * kc;
-    for (int i = tid * 4; i < cells; i += NT_W * 4)
-        *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
-    __syncthreads();
-
-    if (vec_in && rn == R) {
-        // a thread takes 4 consecutive neurons of one batch row: three 16-byte loads, then the
-        // eight x gathers (all from one 4*K-byte row), then the LDS adds
-        const int qpr = R >> 2;   // quads per row
-        const int64_t items = (int64_t)N * qpr;
-        for (int64_t it = tid; it < items; it += NT_W) {
-            const int n = (int)(it / qpr), r0 = (int)(it - (int64_t)n * qpr) * 4;
-            const int64_t o = (int64_t)n * M + m0 + r0;
-            const float4 g = *reinterpret_cast<const float4 *>(grad + o);
-            const int4 i1 = *reinterpret_cast<const int4 *>(argmax + o);
-            const int4 i2 = *reinterpret_cast<const int4 *>(argmin + o);
-            const float gv[4] = {g.x, g.y, g.z, g.w};
-            const int a1[4] = {i1.x - k0, i1.y - k0, i1.z - k0, i1.w - k0};
-            const int a2[4] = {i2.x - k0, i2.y - k0, i2.z - k0, i2.w - k0};
-            const float *xr = x + (int64_t)n * ldx + k0;
-            float x1[4], x2[4];
+    const float gv[4] = {g.x, g.y, g.z, g.w};
+    const int a1[4] = {i1.x - k0, i1.y - k0, i1.z - k0, i1.w - k0};
+    const int a2[4] = {i2.x - k0, i2.y - k0, i2.z - k0, i2.w - k0};
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                x1[u] = (unsigned)a1[u] < (unsigned)kn ? xr[a1[u]] : 0.0f;
-                x2[u] = (unsigned)a2[u] < (unsigned)kn ? xr[a2[u]] : 0.0f;
-            }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int r = r0 + u;
-                if ((unsigned)a1[u] < (unsigned)kn)
-                    lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a1[u] : (a1[u] << log2r) + r], x1[u] * gv[u]);
-                if ((unsigned)a2[u] < (unsigned)kn)
-                    lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a2[u] : (a2[u] << log2r) + r], x2[u] * gv[u]);
-            }
-        }
-    } else {
-        const int64_t pairs = (int64_t)N << log2r;
-        for (int64_t pi = tid; pi < pairs; pi += NT_W) {
-            const int n = (int)(pi >> log2r), r = (int)(pi & (R - 1));
-            if (r >= rn) continue;
-            const int64_t o = (int64_t)n * M + m0 + r;
-            const float g = grad[o];
-            const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
-            const float *xr = x + (int64_t)n * ldx + k0;
-            if ((unsigned)a1 < (unsigned)kn)
-                lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r], xr[a1] * g);
-            if ((unsigned)a2 < (unsigned)kn)
-                lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r], xr[a2] * g);
-        }
+    for (int u = 0; u < 4; ++u) {
+        const int r = r0 + u;
+        if ((unsigned)a1[u] < (unsigned)kn)
+            lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a1[u] : (a1[u] << log2r) + r], x1[u] * gv[u]);
+        if ((unsigned)a2[u] < (unsigned)kn)
+            lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a2[u] : (a2[u] << log2r) + r], x2[u] * gv[u]);
     }
-    __syncthreads();
+}
 
+__device__ __forceinline__ void gather_quad(const float *xr, const int4 &i1, const int4 &i2, int k0, int kn,
+                                            float (&x1)[4], float (&x2)[4])
+{
+    const int a1[4] = {i1.x - k0, i1.y - k0, i1.z - k0, i1.w - k0};
+    const int a2[4] = {i2.x - k0, i2.y - k0, i2.z - k0, i2.w - k0};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        x1[u] = (unsigned)a1[u] < (unsigned)kn ? xr[a1[u]] : 0.0f;
+        x2[u] = (unsigned)a2[u] < (unsigned)kn ? xr[a2[u]] : 0.0f;
+    }
+}
+
+// Stores the slab histogram to w_grad.
+template <int LAYOUT>
+__device__ __forceinline__ void store_slab(const float *hist, float *__restrict__ w_grad, int tid, int m0,
+                                           int k0, int rn, int kn, int kc, int log2r, int K, int M,
+                                           int vec_out)
+{
+    const int R = 1 << log2r;
     if (LAYOUT == MAM_W_MK) {
         if (vec_out) {  // K, k0 and kc are multiples of 4 and w_grad is 16-byte aligned
             const int q = kn >> 2;
@@ -172,6 +142,109 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
             if (r < rn) w_grad[(int64_t)(k0 + kk) * M + m0 + r] = hist[e];
         }
     }
+}
+
+// Fast path (M a multiple of 4, 16-byte aligned grad / argmax / argmin).  A thread's unit of work
+// is one batch row x 4 consecutive neurons: three 16-byte loads, eight x gathers from one row,
+// eight LDS adds.  A workgroup walks `tiles_per_wg` consecutive slabs and software-pipelines them:
+// the index loads of the next slab are issued before the current slab is streamed out, and the x
+// gathers are in flight while the histogram is cleared, so the scatter phase's latency chain
+// (index load -> gather -> LDS add) overlaps the store phase instead of alternating with it.
+template <int LAYOUT>
+__global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
+    const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
+    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
+    float *__restrict__ w_grad, int N, int K, int M, int log2r, int kc, int vec_out, int mtiles,
+    int tiles_per_wg)
+{
+    extern __shared__ float hist[];
+    const int tid = threadIdx.x;
+    const int R = 1 << log2r;
+    const int qpr = R >> 2;
+    const int64_t items = (int64_t)N * qpr;
+    const int k0 = blockIdx.y * kc;
+    const int kn = (K - k0) < kc ? (K - k0) : kc;
+    const int first = xcd_remap(blockIdx.x, gridDim.x) * tiles_per_wg;
+
+    // this thread's first item of a slab: row n_first, neurons m0 + r_first .. +3
+    const int n_first = tid / qpr, r_first = (tid - n_first * qpr) * 4;
+    float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
+    int4 i1 = make_int4(-1, -1, -1, -1), i2 = make_int4(-1, -1, -1, -1);
+    bool have = false;
+    auto load_first = [&](int m0) {
+        have = tid < items && m0 + r_first < M;
+        if (have) {
+            const int64_t o = (int64_t)n_first * M + m0 + r_first;
+            g = *reinterpret_cast<const float4 *>(grad + o);
+            i1 = *reinterpret_cast<const int4 *>(argmax + o);
+            i2 = *reinterpret_cast<const int4 *>(argmin + o);
+        }
+    };
+    if (first < mtiles) load_first(first * R);
+
+    for (int t = 0; t < tiles_per_wg; ++t) {
+        const int mt = first + t;
+        if (mt >= mtiles) break;
+        const int m0 = mt * R;
+        const int rn = (M - m0) < R ? (M - m0) : R;
+        float x1[4], x2[4];
+        if (have) gather_quad(x + (int64_t)n_first * ldx + k0, i1, i2, k0, kn, x1, x2);
+        for (int i = tid * 4; i < R * kc; i += NT_W * 4)
+            *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
+        __syncthreads();
+        if (have) scatter_quad<LAYOUT>(hist, g, i1, i2, x1, x2, r_first, k0, kn, kc, log2r);
+        for (int64_t it = tid + NT_W; it < items; it += NT_W) {
+            const int n = (int)(it / qpr), r0 = (int)(it - (int64_t)n * qpr) * 4;
+            if (m0 + r0 >= M) continue;
+            const int64_t o = (int64_t)n * M + m0 + r0;
+            const float4 gg = *reinterpret_cast<const float4 *>(grad + o);
+            const int4 j1 = *reinterpret_cast<const int4 *>(argmax + o);
+            const int4 j2 = *reinterpret_cast<const int4 *>(argmin + o);
+            float y1[4], y2[4];
+            gather_quad(x + (int64_t)n * ldx + k0, j1, j2, k0, kn, y1, y2);
+            scatter_quad<LAYOUT>(hist, gg, j1, j2, y1, y2, r0, k0, kn, kc, log2r);
+        }
+        __syncthreads();
+        if (t + 1 < tiles_per_wg && mt + 1 < mtiles) load_first(m0 + R);
+        store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out);
+        __syncthreads();
+    }
+}
+
+// Generic path: any M, any alignment; one (batch row, neuron) pair per thread and trip.
+template <int LAYOUT>
+__global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
+    const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
+    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
+    float *__restrict__ w_grad, int N, int K, int M, int log2r, int kc, int vec_out)
+{
+    extern __shared__ float hist[];
+    const int tid = threadIdx.x;
+    const int R = 1 << log2r;
+    const int mt = xcd_remap(blockIdx.x, gridDim.x);
+    const int m0 = mt * R;
+    const int k0 = blockIdx.y * kc;
+    const int rn = (M - m0) < R ? (M - m0) : R;
+    const int kn = (K - k0) < kc ? (K - k0) : kc;
+
+    for (int i = tid * 4; i < R * kc; i += NT_W * 4)
+        *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
+    __syncthreads();
+    const int64_t pairs = (int64_t)N << log2r;
+    for (int64_t pi = tid; pi < pairs; pi += NT_W) {
+        const int n = (int)(pi >> log2r), r = (int)(pi & (R - 1));
+        if (r >= rn) continue;
+        const int64_t o = (int64_t)n * M + m0 + r;
+        const float g = grad[o];
+        const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
+        const float *xr = x + (int64_t)n * ldx + k0;
+        if ((unsigned)a1 < (unsigned)kn)
+            lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r], xr[a1] * g);
+        if ((unsigned)a2 < (unsigned)kn)
+            lds_add(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r], xr[a2] * g);
+    }
+    __syncthreads();
+    store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out);
 }
 
 // LDS a workgroup may use for a histogram, in floats.  gfx950 has 160 KiB per CU; above
@@ -201,12 +274,14 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         if (rc != MAM_OK) return rc;
     }
     if (w_grad) {
-        // (M,K): 4 whole-K rows in 64 KiB, so two workgroups share a CU and one's scatter phase
-        // overlaps the other's store phase.  (K,M): 32 columns x 1024 k in 128 KiB.
+        // (M,K): 4 whole-K rows in 64 KiB, so two workgroups share a CU.  (K,M): 32 columns x
+        // 1024 k in 128 KiB.
         static const int big = lds_budget_floats((const void *)mam_bwd_w_kernel<LAYOUT>);
+        static const int big2 = lds_budget_floats((const void *)mam_bwd_w_vec_kernel<LAYOUT>);
         const int log2r = LAYOUT == MAM_W_MK ? 2 : 5;
         const int R = 1 << log2r;
-        const int budget = LAYOUT == MAM_W_MK ? 64 * 1024 / 4 : big;
+        const int lds_cap = big < big2 ? big : big2;
+        const int budget = LAYOUT == MAM_W_MK ? (R * 4096 < lds_cap ? R * 4096 : lds_cap) : lds_cap;
         int kc = budget / R;
         if (K < kc) kc = (int)((K + 3) / 4 * 4);
         const int64_t mtiles = ceil_div(M, R), ktiles = ceil_div(K, kc);
@@ -214,9 +289,20 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         const int vec_out = (K % 4 == 0) && ((uintptr_t)w_grad % 16 == 0);
         const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
                            ((uintptr_t)argmin % 16 == 0);
-        hipLaunchKernelGGL((mam_bwd_w_kernel<LAYOUT>), dim3((unsigned)mtiles, (unsigned)ktiles),
-                           dim3(NT_W), (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax,
-                           argmin, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out, vec_in);
+        if (vec_in) {
+            // slabs per workgroup: enough workgroups for two per CU, the rest goes into pipelining
+            int tpw = (int)(mtiles * ktiles / (2 * kNumCU));
+            if (tpw < 1) tpw = 1;
+            if (tpw > 8) tpw = 8;
+            hipLaunchKernelGGL((mam_bwd_w_vec_kernel<LAYOUT>),
+                               dim3((unsigned)ceil_div(mtiles, tpw), (unsigned)ktiles), dim3(NT_W),
+                               (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax, argmin, w_grad,
+                               (int)N, (int)K, (int)M, log2r, kc, vec_out, (int)mtiles, tpw);
+        } else {
+            hipLaunchKernelGGL((mam_bwd_w_kernel<LAYOUT>), dim3((unsigned)mtiles, (unsigned)ktiles),
+                               dim3(NT_W), (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax,
+                               argmin, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out);
+        }
         rc = check_launch("mam_bwd_w_kernel");
     }
     return rc;

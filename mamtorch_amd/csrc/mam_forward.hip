@@ -169,7 +169,11 @@ template <class NM>
 __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps,
                                              int lane, NM nm_of)
 {
-    // rounds are unrolled so that the loads of all of them are in flight together
+    // Two passes over the rounds, both unrolled: every load of every round first (stores
+    // between them would pin the loads in program order), then the stores.
+    float r_sum[RES_ROUNDS], r_wmax[RES_ROUNDS], r_wmin[RES_ROUNDS];
+    int r_imax[RES_ROUNDS], r_imin[RES_ROUNDS];
+    int64_t r_out[RES_ROUNDS];
 #pragma unroll
     for (int r = 0; r < RES_ROUNDS; ++r) {
         const int task = r * TPR + lane / LPT;
@@ -203,18 +207,26 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
         const int idx = g * G + key;
         // lanes of the max task and of the min task of one output are LPT apart
         const float val_min = __shfl_xor(val, LPT);
-        const int idx_min = __shfl_xor(idx, LPT);
-        const float wsel_min = __shfl_xor(wsel, LPT);
-        if (ext == 0 && sub == 0 && valid) {
-            float sum = val + val_min;
-            if (p.bias) sum = sum + p.bias[m];
-            const int64_t o = (int64_t)n * p.M + m;
-            p.c[o] = sum;
-            p.argmax[o] = idx;
-            p.argmin[o] = idx_min;
+        float sum = val + val_min;
+        if (p.bias) sum = sum + p.bias[m];
+        r_sum[r] = sum;
+        r_imax[r] = idx;
+        r_imin[r] = __shfl_xor(idx, LPT);
+        r_wmax[r] = wsel;
+        r_wmin[r] = __shfl_xor(wsel, LPT);
+        r_out[r] = (ext == 0 && sub == 0 && valid) ? (int64_t)n * p.M + m : (int64_t)-1;
+    }
+    const int64_t nm = (int64_t)p.N * p.M;
+#pragma unroll
+    for (int r = 0; r < RES_ROUNDS; ++r) {
+        const int64_t o = r_out[r];
+        if (o >= 0) {
+            p.c[o] = r_sum[r];
+            p.argmax[o] = r_imax[r];
+            p.argmin[o] = r_imin[r];
             if (p.wsel) {
-                p.wsel[o] = wsel;
-                p.wsel[(int64_t)p.N * p.M + o] = wsel_min;
+                p.wsel[o] = r_wmax[r];
+                p.wsel[nm + o] = r_wmin[r];
             }
         }
     }
@@ -578,7 +590,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 
 // Combines split-K partials in ascending k order (strict comparisons keep the earliest
 // group on ties), then resolves indices / zero signs exactly as the single-pass epilogue.
-template <int LAYOUT, bool ARGS>
+template <int LAYOUT, bool ARGS, bool COOP>
 __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
 {
     // A workgroup owns a 16 x 16 patch of c.  Resolving re-reads G weights of row m per output,
@@ -620,7 +632,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
             }
         }
     }
-    if (ARGS && p.coop) {
+    if (COOP) {
         const int lane = threadIdx.x & 63;
         const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
         vals_s[wave][0][lane] = vmax;
@@ -637,10 +649,9 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
                          n = n < p.N ? n : p.N - 1;
                          m = m < p.M ? m : p.M - 1;
                      });
-        return;
+    } else if (live) {
+        finish<LAYOUT, ARGS>(p, n_own, m_own, vmax, vmin, gmax, gmin);
     }
-    if (!live) return;
-    finish<LAYOUT, ARGS>(p, n_own, m_own, vmax, vmin, gmax, gmin);
 }
 
 // How many K ranges to split into so that at least two workgroups reach every CU.
@@ -721,10 +732,12 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     if (rc != MAM_OK) return rc;
     if (p.splits > 1) {
         const unsigned mb = (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
-        if (w_layout == MAM_W_MK)
-            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS>), dim3(mb), dim3(256), 0, st, p);
+        if (ARGS && p.coop)
+            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS, ARGS>), dim3(mb), dim3(256), 0, st, p);
+        else if (w_layout == MAM_W_MK)
+            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS, false>), dim3(mb), dim3(256), 0, st, p);
         else
-            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_KM, ARGS>), dim3(mb), dim3(256), 0, st, p);
+            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_KM, ARGS, false>), dim3(mb), dim3(256), 0, st, p);
         rc = check_launch("mam_fwd_merge_kernel");
     }
     return rc;

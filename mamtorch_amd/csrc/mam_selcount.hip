@@ -2,29 +2,36 @@
 // into (M, K) int32 counters.  Replaces FullyConnected.update_selection_count
 // (mamtorch/nn/v4/fullyconnected.py:114-129), which runs two advanced-index "+= 1" statements.
 //
-// MAM_COUNT_REFERENCE reproduces that code literally: an advanced-index "+= 1" does not
-// accumulate duplicate indices, and both statements write max_selection_count, so per call a
-// cell gains 1 if any batch row picked it as argmax plus 1 if any row picked it as argmin.  A
-// workgroup owns R consecutive neurons, marks picks in two LDS bitmaps (ds_or), then walks the
-// set bits and applies plain read-modify-writes to its own rows: the counters are touched only
-// where something was picked, and no global atomics are needed.
+// A workgroup owns R = 4 consecutive neurons x kc columns of the counters.  Picks are collected
+// in LDS words that hold two 16-bit fields (low: argmax, high: argmin), then the slab is streamed
+// back with 16-byte read-modify-writes that skip chunks nothing was picked in.  At training batch
+// sizes nearly every cache line of the counters holds a pick, so this is a coalesced pass over
+// the slab; at small N*M it degenerates to a sparse update.  No global atomics.
 //
-// MAM_COUNT_HITS counts every pick with the same ownership scheme and LDS counters.
+// MAM_COUNT_HITS: the fields are counters (LDS atomic add; the batch is walked in chunks of 32768
+// rows so that neither field overflows).
+// MAM_COUNT_REFERENCE reproduces the module literally: an advanced-index "+= 1" does not
+// accumulate duplicate indices, and both statements write max_selection_count, so per call a cell
+// gains 1 if any batch row picked it as argmax plus 1 if any row picked it as argmin.  The fields
+// are flags (LDS atomic or) and max_count receives flag(max) + flag(min); min_count is untouched.
 #include "mam_common.h"
 
 namespace mam {
 namespace selcount {
 
-constexpr int NT = 256;
 
-// Hit counting: a workgroup owns R neurons x kc columns of both counters.  Picks are counted in
-// LDS words holding two 16-bit counters (low half: argmax hits, high half: argmin hits; the batch
-// is walked in chunks of 32768 rows so that neither half overflows), then only the cells that
-// were hit are read-modify-written in HBM.
 constexpr int NT_H = 512;
+
+template <int MODE>
+__device__ __forceinline__ void mark(uint32_t *word, uint32_t field)
+{
+    if (MODE == MAM_COUNT_HITS) atomicAdd(word, field); else atomicOr(word, field);
+}
+
 constexpr int ROWS_PER_PASS = 32768;
 
-__global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ argmax,
+template <int MODE>
+__global__ __launch_bounds__(NT_H) void count_kernel(const int32_t *__restrict__ argmax,
                                                     const int32_t *__restrict__ argmin,
                                                     int32_t *__restrict__ max_count,
                                                     int32_t *__restrict__ min_count, int N, int M,
@@ -37,11 +44,12 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
     const int k0 = blockIdx.y * kc;
     const int rn = (M - m0) < R ? (M - m0) : R;
     const int kn = (K - k0) < kc ? (K - k0) : kc;
-    for (int n0 = 0; n0 < N; n0 += ROWS_PER_PASS) {
-        const int nn = (N - n0) < ROWS_PER_PASS ? (N - n0) : ROWS_PER_PASS;
+    const int rows_per_pass = MODE == MAM_COUNT_HITS ? ROWS_PER_PASS : N;   // flags cannot overflow
+    for (int n0 = 0; n0 < N; n0 += rows_per_pass) {
+        const int nn = (N - n0) < rows_per_pass ? (N - n0) : rows_per_pass;
         for (int i = tid; i < R * kc; i += NT_H) cnt[i] = 0u;
         __syncthreads();
-        if (vec_in && rn == R) {
+        if (vec_in && rn == R && R >= 4) {
             const int qpr = R >> 2;
             const int items = nn * qpr;
             for (int it = tid; it < items; it += NT_H) {
@@ -53,8 +61,8 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
                 const int a2[4] = {i2.x - k0, i2.y - k0, i2.z - k0, i2.w - k0};
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    if ((unsigned)a1[u] < (unsigned)kn) atomicAdd(&cnt[(r0 + u) * kc + a1[u]], 1u);
-                    if ((unsigned)a2[u] < (unsigned)kn) atomicAdd(&cnt[(r0 + u) * kc + a2[u]], 0x10000u);
+                    if ((unsigned)a1[u] < (unsigned)kn) mark<MODE>(&cnt[(r0 + u) * kc + a1[u]], 1u);
+                    if ((unsigned)a2[u] < (unsigned)kn) mark<MODE>(&cnt[(r0 + u) * kc + a2[u]], 0x10000u);
                 }
             }
         } else {
@@ -64,8 +72,8 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
                 if (r >= rn) continue;
                 const int64_t o = (int64_t)n * M + m0 + r;
                 const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
-                if ((unsigned)a1 < (unsigned)kn) atomicAdd(&cnt[r * kc + a1], 1u);
-                if ((unsigned)a2 < (unsigned)kn) atomicAdd(&cnt[r * kc + a2], 0x10000u);
+                if ((unsigned)a1 < (unsigned)kn) mark<MODE>(&cnt[r * kc + a1], 1u);
+                if ((unsigned)a2 < (unsigned)kn) mark<MODE>(&cnt[r * kc + a2], 0x10000u);
             }
         }
         __syncthreads();
@@ -88,6 +96,16 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
                         const int r = e / q, c4 = e - r * q;
                         v[u] = *reinterpret_cast<const uint4 *>(&cnt[r * kc + c4 * 4]);
                         cell[u] = (int64_t)(m0 + r) * K + k0 + c4 * 4;
+                    }
+                }
+                if (MODE == MAM_COUNT_REFERENCE) {
+                    // both flags land in max_count: fold them into the low field
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        v[u].x = (v[u].x & 1u) + (v[u].x >> 16);
+                        v[u].y = (v[u].y & 1u) + (v[u].y >> 16);
+                        v[u].z = (v[u].z & 1u) + (v[u].z >> 16);
+                        v[u].w = (v[u].w & 1u) + (v[u].w >> 16);
                     }
                 }
 #pragma unroll
@@ -114,7 +132,8 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
         } else {
             for (int e = tid; e < rn * kn; e += NT_H) {
                 const int r = e / kn, kk = e - r * kn;
-                const uint32_t v = cnt[r * kc + kk];
+                uint32_t v = cnt[r * kc + kk];
+                if (MODE == MAM_COUNT_REFERENCE) v = (v & 1u) + (v >> 16);
                 if (v) {
                     const int64_t cell = (int64_t)(m0 + r) * K + k0 + kk;
                     if (v & 0xffffu) max_count[cell] += (int)(v & 0xffffu);
@@ -123,42 +142,6 @@ __global__ __launch_bounds__(NT_H) void hits_kernel(const int32_t *__restrict__ 
             }
         }
         __syncthreads();
-    }
-}
-
-__global__ __launch_bounds__(NT) void reference_kernel(const int32_t *__restrict__ argmax,
-                                                       const int32_t *__restrict__ argmin,
-                                                       int32_t *__restrict__ max_count, int N, int M,
-                                                       int K, int log2r, int words)
-{
-    extern __shared__ uint32_t bits[];  // [2][R][words]
-    const int tid = threadIdx.x;
-    const int R = 1 << log2r;
-    const int m0 = xcd_remap(blockIdx.x, gridDim.x) * R;
-    const int rn = (M - m0) < R ? (M - m0) : R;
-    const int plane = R * words;
-    for (int i = tid; i < 2 * plane; i += NT) bits[i] = 0u;
-    __syncthreads();
-    const int64_t pairs = (int64_t)N << log2r;
-    for (int64_t pi = tid; pi < pairs; pi += NT) {
-        const int n = (int)(pi >> log2r), r = (int)(pi & (R - 1));
-        if (r >= rn) continue;
-        const int64_t o = (int64_t)n * M + m0 + r;
-        const int a1 = argmax[o], a2 = argmin[o];
-        if ((unsigned)a1 < (unsigned)K) atomicOr(&bits[r * words + (a1 >> 5)], 1u << (a1 & 31));
-        if ((unsigned)a2 < (unsigned)K) atomicOr(&bits[plane + r * words + (a2 >> 5)], 1u << (a2 & 31));
-    }
-    __syncthreads();
-    for (int e = tid; e < rn * words; e += NT) {
-        const int r = e / words, wi = e - r * words;
-        const uint32_t b1 = bits[r * words + wi], b2 = bits[plane + r * words + wi];
-        uint32_t u = b1 | b2;
-        int32_t *row = max_count + (int64_t)(m0 + r) * K + wi * 32;
-        while (u) {
-            const int b = __builtin_ctz(u);
-            u &= u - 1;
-            row[b] += (int)((b1 >> b) & 1u) + (int)((b2 >> b) & 1u);
-        }
     }
 }
 
@@ -179,31 +162,25 @@ extern "C" int mam_selection_count(const int32_t *argmax, const int32_t *argmin,
     if (N > INT32_MAX / 2 || K > INT32_MAX / 2 || M > INT32_MAX / 2)
         return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (mode == MAM_COUNT_HITS) {
-        // 4 whole-K rows of packed counters in 64 KiB: two workgroups per CU
-        const int budget = 64 * 1024 / 4;
-        const int log2r = 2;
-        const int R = 1 << log2r;
-        int kc = budget / R;
-        if (K < kc) kc = (int)((K + 3) / 4 * 4);
-        const int64_t ktiles = ceil_div(K, kc);
-        const int vec = (K % 4 == 0) && ((uintptr_t)max_count % 16 == 0) && ((uintptr_t)min_count % 16 == 0);
-        const int vec_in = (M % 4 == 0) && ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0);
-        if (ktiles > 65535) return fail(MAM_ERR_UNSUPPORTED, "K too large for the selection-count grid");
-        hipLaunchKernelGGL(selcount::hits_kernel, dim3((unsigned)ceil_div(M, R), (unsigned)ktiles),
-                           dim3(selcount::NT_H), (size_t)R * kc * 4, st, argmax, argmin, max_count,
-                           min_count, (int)N, (int)M, (int)K, log2r, kc, vec, vec_in);
-        return check_launch("selcount::hits_kernel");
-    }
-    const int words = (int)ceil_div(K, 32);
-    // two bitmaps of R rows in at most 48 KiB of LDS
-    int log2r = 5;
-    while (log2r > 0 && (int64_t)2 * (1 << log2r) * words * 4 > 48 * 1024) --log2r;
-    if ((int64_t)2 * (1 << log2r) * words * 4 > 48 * 1024)
-        return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds the bitmap capacity (196608)", (long long)K);
+    // 4 whole-K rows of packed fields in 64 KiB: two workgroups per CU
+    const int budget = 64 * 1024 / 4;
+    const int log2r = 2;
     const int R = 1 << log2r;
-    hipLaunchKernelGGL(selcount::reference_kernel, dim3((unsigned)ceil_div(M, R)), dim3(selcount::NT),
-                       (size_t)2 * R * words * 4, st, argmax, argmin, max_count, (int)N, (int)M, (int)K,
-                       log2r, words);
-    return check_launch("selcount::reference_kernel");
+    int kc = budget / R;
+    if (K < kc) kc = (int)((K + 3) / 4 * 4);
+    const int64_t ktiles = ceil_div(K, kc);
+    if (ktiles > 65535) return fail(MAM_ERR_UNSUPPORTED, "K too large for the selection-count grid");
+    const int vec = (K % 4 == 0) && ((uintptr_t)max_count % 16 == 0) &&
+                    (mode == MAM_COUNT_REFERENCE || (uintptr_t)min_count % 16 == 0);
+    const int vec_in = (M % 4 == 0) && ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0);
+    const dim3 grid((unsigned)ceil_div(M, R), (unsigned)ktiles);
+    if (mode == MAM_COUNT_HITS)
+        hipLaunchKernelGGL(selcount::count_kernel<MAM_COUNT_HITS>, grid, dim3(selcount::NT_H),
+                           (size_t)R * kc * 4, st, argmax, argmin, max_count, min_count, (int)N, (int)M,
+                           (int)K, log2r, kc, vec, vec_in);
+    else
+        hipLaunchKernelGGL(selcount::count_kernel<MAM_COUNT_REFERENCE>, grid, dim3(selcount::NT_H),
+                           (size_t)R * kc * 4, st, argmax, argmin, max_count, min_count, (int)N, (int)M,
+                           (int)K, log2r, kc, vec, vec_in);
+    return check_launch("selcount::count_kernel");
 }
