@@ -318,7 +318,7 @@ static_assert(TILE_FLOATS % 256 == 0 && (BN * LDK) % 256 == 0, "tile must be who
 // Per-lane source offsets of a wave's loads live in LDS ([load][thread]): they are needed once
 // per tile, and a register spilled to scratch would be reloaded through the same counter that
 // tracks the loads in flight.
-__device__ __forceinline__ void dma_tile(const float *xt, const float *wt, float *tile, int wave,
+__device__ __forceinline__ void dma_tile(const char *xt, const char *wt, float *tile, int wave,
                                          const uint32_t *doff, bool x_only)
 {
 #pragma unroll
@@ -328,7 +328,9 @@ __device__ __forceinline__ void dma_tile(const float *xt, const float *wt, float
         inst = inst < DMA_INSTR ? inst : DMA_INSTR - 1;
         if (x_only && t * (NT / 64) >= DMA_X_INSTR) break;
         if (x_only) inst = inst < DMA_X_INSTR ? inst : DMA_X_INSTR - 1;
-        const float *src = (inst < DMA_X_INSTR ? xt : wt) + doff[t * NT];
+        // uniform 64-bit base + 32-bit lane offset: the scalar-base form of the load, one
+        // address register per load
+        const char *src = (inst < DMA_X_INSTR ? xt : wt) + (uint64_t)doff[t * NT];
         __builtin_amdgcn_global_load_lds(
             (const __attribute__((address_space(1))) void *)src,
             (__attribute__((address_space(3))) void *)(tile + inst * 256), 16, 0, 0);
@@ -339,15 +341,15 @@ __device__ __forceinline__ void dma_tile(const float *xt, const float *wt, float
 // unrolled so that the running extremes ping-pong between two register sets: the value before
 // the group stays readable for the "did it improve" test without a copy.
 template <bool ARGS>
-__device__ __forceinline__ void compute_tile(const float *tile, int tx, int ty, uint32_t grel0,
+__device__ __forceinline__ void compute_tile(const float *tile, int tx, int ty, int grel0,
                                              float (&vmax)[TI][TJ], float (&vmin)[TI][TJ],
-                                             uint32_t (&gsel)[TI][TJ])
+                                             int (&gmax)[TI][TJ], int (&gmin)[TI][TJ])
 {
     const float (*xs)[LDK] = reinterpret_cast<const float (*)[LDK]>(tile);
     const float (*ws)[LDK] = reinterpret_cast<const float (*)[LDK]>(tile + BN * LDK);
 #pragma unroll
     for (int gg = 0; gg < KT / G; ++gg) {
-        const uint32_t grel = grel0 + gg;
+        const int grel = grel0 + gg;
         float xv[TI][G];
 #pragma unroll
         for (int i = 0; i < TI; ++i)
@@ -377,17 +379,10 @@ __device__ __forceinline__ void compute_tile(const float *tile, int tx, int ty, 
                     lo = __builtin_fminf(__builtin_fminf(lo, a), b);   // v_min3_f32
                 }
                 if (ARGS) {
-                    // gsel.lo16 = (hi > om) ? grel : gsel.lo16 ; gsel.hi16 likewise for the min.
-                    // One compare and one sub-dword conditional move per extreme: the select
-                    // picks a 16-bit word of each source and writes one word of gsel.
-                    asm("v_cmp_gt_f32 vcc, %1, %2\n\t"
-                        "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_0 dst_unused:UNUSED_PRESERVE "
-                        "src0_sel:WORD_0 src1_sel:WORD_0"
-                        : "+v"(gsel[i][j]) : "v"(hi), "v"(om), "v"(grel) : "vcc");
-                    asm("v_cmp_lt_f32 vcc, %1, %2\n\t"
-                        "v_cndmask_b32_sdwa %0, %0, %3, vcc dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE "
-                        "src0_sel:WORD_1 src1_sel:WORD_0"
-                        : "+v"(gsel[i][j]) : "v"(lo), "v"(on), "v"(grel) : "vcc");
+                    // one compare + one select per extreme and group, left to the compiler to
+                    // place: issued back to back they stall on the condition mask
+                    gmax[i][j] = (hi > om) ? grel : gmax[i][j];
+                    gmin[i][j] = (lo < on) ? grel : gmin[i][j];
                 }
                 vmax[i][j] = hi;
                 vmin[i][j] = lo;
@@ -427,16 +422,16 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
     const int ntiles = (ke - kb + KT - 1) / KT;
 
     float vmax[TI][TJ], vmin[TI][TJ];
-    // group of the running max in bits 0..15, of the running min in bits 16..31, both counted
-    // from the first group of this workgroup's k range
-    uint32_t gsel[TI][TJ];
+    // groups of the running max / min, counted from the first group of this workgroup's k range
+    int gmax[TI][TJ], gmin[TI][TJ];
 #pragma unroll
     for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int j = 0; j < TJ; ++j) {
             vmax[i][j] = -__builtin_inff();
             vmin[i][j] = __builtin_inff();
-            gsel[i][j] = 0u;
+            gmax[i][j] = 0;
+            gmin[i][j] = 0;
         }
 
     // ---- staging ----
@@ -461,10 +456,10 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
         uint32_t off;
         if (row < BN) {
             const int r = ((row0 + row) < p.N ? (row0 + row) : (p.N - 1)) - row0;
-            off = (uint32_t)(r * (int)p.ldx + ch * 4);
+            off = (uint32_t)(r * (int)p.ldx + ch * 4) * 4u;
         } else {
             const int c = ((col0 + row - BN) < p.M ? (col0 + row - BN) : (p.M - 1)) - col0;
-            off = (uint32_t)(c * (int)p.ldw + ch * 4);
+            off = (uint32_t)(c * (int)p.ldw + ch * 4) * 4u;
         }
         doff_s[t * NT + tid] = off;
     }
@@ -479,34 +474,48 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
         }
     }
 
-    // stage tile `t` into `dst`; returns after the loads are ISSUED (direct-to-LDS) or DONE
-    auto stage = [&](float *dst, int t) {
-        const int k0 = kb + t * KT;
-        float (*xs)[LDK] = reinterpret_cast<float (*)[LDK]>(dst);
-        float (*ws)[LDK] = reinterpret_cast<float (*)[LDK]>(dst + BN * LDK);
-        if (fast && k0 + KT <= ke) {
-            if (LAYOUT == MAM_W_MK) {
-                dma_tile(xbase + k0, wbase + k0, dst, wave, doff, false);
-            } else {
-                // x by direct-to-LDS, w through registers
-                dma_tile(xbase + k0, xbase + k0, dst, wave, doff, true);
-                stage_w_km_fast(wbase + (int64_t)k0 * p.ldw, ws, tid, wo);
+    // Tiles that take the direct-to-LDS path: double-buffered, loads one tile ahead of the
+    // arithmetic, nothing but the running extremes, the operands and three addresses live.
+    int t0 = 0;
+    if (LAYOUT == MAM_W_MK && fast) {
+        const int full = (ke - kb) / KT;
+        if (full > 0) {
+            const char *xk = reinterpret_cast<const char *>(xbase + kb);
+            const char *wk = reinterpret_cast<const char *>(wbase + kb);
+            dma_tile(xk, wk, tile_a, wave, doff, false);
+            __syncthreads();
+            for (int t = 0; t < full; t += 2) {
+                xk += KT * sizeof(float);
+                wk += KT * sizeof(float);
+                if (t + 1 < full) dma_tile(xk, wk, tile_b, wave, doff, false);
+                compute_tile<ARGS>(tile_a, tx, ty, t * (KT / G), vmax, vmin, gmax, gmin);
+                __syncthreads();
+                if (t + 1 >= full) break;
+                xk += KT * sizeof(float);
+                wk += KT * sizeof(float);
+                if (t + 2 < full) dma_tile(xk, wk, tile_a, wave, doff, false);
+                compute_tile<ARGS>(tile_b, tx, ty, (t + 1) * (KT / G), vmax, vmin, gmax, gmin);
+                __syncthreads();
             }
+            t0 = full;
+        }
+    }
+    // Everything else, one tile at a time: the ragged k tail, unaligned views, and the (K,M)
+    // layout, whose w goes through registers because it has to be transposed.
+#pragma unroll 1
+    for (int t = t0; t < ntiles; ++t) {
+        const int k0 = kb + t * KT;
+        float (*xs)[LDK] = reinterpret_cast<float (*)[LDK]>(tile_a);
+        float (*ws)[LDK] = reinterpret_cast<float (*)[LDK]>(tile_a + BN * LDK);
+        if (LAYOUT == MAM_W_KM && fast && k0 + KT <= ke) {
+            const char *xk = reinterpret_cast<const char *>(xbase + k0);
+            dma_tile(xk, xk, tile_a, wave, doff, true);
+            stage_w_km_fast(wbase + (int64_t)k0 * p.ldw, ws, tid, wo);
         } else {
             stage_tile_generic<LAYOUT>(p, xs, ws, tid, row0, col0, k0, ke);
         }
-    };
-
-    stage(tile_a, 0);
-    __syncthreads();
-    for (int t = 0; t < ntiles; t += 2) {
-        // tile t from buffer A while tile t+1 lands in buffer B
-        if (t + 1 < ntiles) stage(tile_b, t + 1);
-        compute_tile<ARGS>(tile_a, tx, ty, (uint32_t)(t * (KT / G)), vmax, vmin, gsel);
         __syncthreads();
-        if (t + 1 >= ntiles) break;
-        if (t + 2 < ntiles) stage(tile_a, t + 2);
-        compute_tile<ARGS>(tile_b, tx, ty, (uint32_t)((t + 1) * (KT / G)), vmax, vmin, gsel);
+        compute_tile<ARGS>(tile_a, tx, ty, t * (KT / G), vmax, vmin, gmax, gmin);
         __syncthreads();
     }
 
@@ -526,8 +535,8 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
             for (int j = 0; j < TJ; ++j) {
                 vals[(j * 2 + 0) * 64 + lane] = vmax[i][j];
                 vals[(j * 2 + 1) * 64 + lane] = vmin[i][j];
-                grps[(j * 2 + 0) * 64 + lane] = g0 + (int)(gsel[i][j] & 0xffffu);
-                grps[(j * 2 + 1) * 64 + lane] = g0 + (int)(gsel[i][j] >> 16);
+                grps[(j * 2 + 0) * 64 + lane] = g0 + gmax[i][j];
+                grps[(j * 2 + 1) * 64 + lane] = g0 + gmin[i][j];
             }
             __syncthreads();
 #pragma unroll 1
@@ -555,7 +564,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
             for (int j = 0; j < TJ; ++j) {
                 stash[(0 * TJ + j) * NT] = vmax[i][j];
                 stash[(1 * TJ + j) * NT] = vmin[i][j];
-                stash[(2 * TJ + j) * NT] = __uint_as_float(gsel[i][j]);
+                stash[(2 * TJ + j) * NT] = __int_as_float(gmax[i][j] | (gmin[i][j] << 16));
             }
             const int n = row0 + ty + 16 * i;
             if (n < p.N) {
@@ -582,7 +591,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
                     const int64_t o = (int64_t)n * p.M + m;
                     base[o] = vmax[i][j];
                     base[nm + o] = vmin[i][j];
-                    if (ARGS) base[2 * nm + o] = __uint_as_float(gsel[i][j]);
+                    if (ARGS) base[2 * nm + o] = __int_as_float(gmax[i][j] | (gmin[i][j] << 16));
                 }
             }
     }
