@@ -27,6 +27,10 @@ N, K, M = 256, 4096, 4096
 VALU_PEAK_TFLOPS = 78.65      # 256 CU x 4 SIMD x 16 lanes x 2 (packed width) x 2.4 GHz, no FMA x2
 VECTOR_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters, each scaled by what the same
+# counter reads for the plain 64 MiB copy below (profiles/hbm_traffic_headline_n256_k4096_m4096.md)
+FORWARD_TRAFFIC_BYTES = {"mam_fwd_kernel": 141.1e6, "mam_fwd_merge_kernel": 167.7e6}
+BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 103.4e6}
 
 
 def make_inputs(torch, dev):
@@ -175,23 +179,27 @@ def main():
         "fwd_bwd_gops": round(triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e9, 2),
         "fwd_bwd_valu_frac": round(3.0 * triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e12 / VALU_PEAK_TFLOPS, 4),
         "roofline": {
-            "kernel": "mam_fwd_kernel<MK,args> (+ split-K merge)",
+            "kernel": "mam_fwd_kernel<MK,args> + mam_fwd_merge_kernel (one mam_fc_forward call)",
             "bound": "valu",
             "achieved": round(fwd_tflops, 3),
             "peak": VALU_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(fwd_tflops / VALU_PEAK_TFLOPS, 4),
             "frac_of_vector_fp32_157.3": round(fwd_tflops / VECTOR_FP32_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": sum(FORWARD_TRAFFIC_BYTES.values()),
+            "traffic_by_kernel": FORWARD_TRAFFIC_BYTES,
+            "algorithmic_bytes": 4 * (N * K + K * M + 4 * N * M),
         },
         "roofline_backward": {
-            "kernel": "mam_bwd_x_kernel + mam_bwd_w_kernel",
+            "kernel": "mam_bwd_x_kernel + mam_bwd_w_vec_kernel",
             "bound": "hbm",
             "achieved": round(bwd_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(bwd_gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": sum(BACKWARD_TRAFFIC_BYTES.values()),
+            "traffic_by_kernel": BACKWARD_TRAFFIC_BYTES,
+            "algorithmic_bytes": bwd_bytes,
         },
     }
     if args.cpu_seconds > 0:
