@@ -1,17 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the MAM fully-connected hot path on one MI355X.
 
-One "step" = one pass of the hot path over one synthetic batch of the headline configuration
-(MAM FullyConnected fp32, batch 256, in = out = 4096): exact forward with argmax/argmin, backward
-(grad_x, grad_W), and selection-count accumulation, launched back to back on one stream through
-the C ABI of libmam_hip.so with all inputs already resident in HBM.
+Default workload ("headline"): one "step" = one pass of the hot path over one synthetic batch of
+MAM FullyConnected fp32, batch 256, in = out = 4096: exact forward with argmax/argmin, backward
+(grad_x, grad_W), and selection-count accumulation (true hit counts), launched back to back on one
+stream through the C ABI of libmam_hip.so with all inputs already resident in HBM.
 
-Prints ONE JSON line.  `value` is N*K*M / t_step in GOPS (one op = one multiply-max-min triple).
-`roofline` describes the dominant kernel (the forward, FP32-VALU bound: 3 fp32 ops per triple
-against 256 CUs x 128 lanes x 2.4 GHz = 78.6 T fp32-op/s, i.e. the 157.3 TFLOP/s vector peak
-without the FMA factor that a (max, min, x) semiring cannot use).  `roofline_backward` gives the
+Prints ONE JSON line.  `value` is (multiply-max-min triples per step) / t_step in GOPS.
+`roofline` describes the dominant kernel: for the dense workloads the forward, FP32-VALU bound
+(3 fp32 ops per triple against 256 CUs x 128 lanes x 2.4 GHz = 78.6 T fp32-op/s, i.e. the
+157.3 TFLOP/s vector peak without the FMA factor that a (max, min, x) semiring cannot use); for
+the CSR-sparse workloads the forward against HBM bandwidth.  `roofline_backward` gives the
 backward's algorithmic bytes over its time against 8 TB/s.  `cpu_baseline` is the pure-PyTorch
 restatement of the reference's CPU path (oracle/torch_port.py) timed on a bounded row sample.
+
+Other workloads (`--workload`), same JSON layout, used for the tables in the design notes:
+  vit_mlp            12608 rows through MAM FC 768->3072 and MAM FC 3072->768, forward + backward
+  inference_m{1024,4096,16384}   batch 16384, in 4096, forward with indices only
+  values_headline    headline shape, values-only forward
+  sparse_d{10,03,01} 4096x4096 weight pruned to 10 % / 3 % / 1 %, batch 256, CSR forward + backward
 """
 import argparse
 import ctypes
@@ -23,61 +30,307 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-N, K, M = 256, 4096, 4096
 VALU_PEAK_TFLOPS = 78.65      # 256 CU x 4 SIMD x 16 lanes x 2 (packed width) x 2.4 GHz, no FMA x2
 VECTOR_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counters, each scaled by what the same
-# counter reads for the plain 64 MiB copy below (profiles/hbm_traffic_headline_n256_k4096_m4096.md)
+# HBM bytes per launch at the headline shape from the FETCH_SIZE / WRITE_SIZE counters, each scaled
+# by what the same counter reads for the plain 64 MiB copy made before the warm-up
+# (profiles/hbm_traffic_headline_n256_k4096_m4096.md)
 FORWARD_TRAFFIC_BYTES = {"mam_fwd_kernel": 141.1e6, "mam_fwd_merge_kernel": 167.7e6}
 BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 103.4e6}
 
-
-def make_inputs(torch, dev):
-    gen = torch.Generator().manual_seed(0)
-    x = torch.randn(N, K, generator=gen)
-    w = (torch.rand(M, K, generator=gen) * 2 - 1) / 64.0   # weight (out, in) ~ U(-1/64, 1/64)
-    g = torch.randn(N, M, generator=gen)
-    return x, w, g
+WORKLOADS = ("headline", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
+             "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01")
 
 
-def cpu_baseline(torch, x, w, g, budget_s):
-    """Times forward + backward of the pure-PyTorch port on the first `rows` batch rows."""
+class Layer:
+    """One dense MAM layer's buffers and its C-ABI calls on the current stream."""
+
+    def __init__(self, torch, capi, lib, dev, x, w, g, want_backward, want_count, values_only=False):
+        self.lib, self.capi = lib, capi
+        self.N, self.K = x.shape
+        self.M = w.shape[0]
+        N, K, M = self.N, self.K, self.M
+        self.x, self.w, self.g = x.to(dev), w.to(dev), None if g is None else g.to(dev)
+        self.values_only = values_only
+        self.c = torch.empty((N, M), dtype=torch.float32, device=dev)
+        if not values_only:
+            self.amax = torch.empty((N, M), dtype=torch.int32, device=dev)
+            self.amin = torch.empty((N, M), dtype=torch.int32, device=dev)
+        if want_backward:
+            self.xg = torch.empty((N, K), dtype=torch.float32, device=dev)
+            self.wg = torch.empty((M, K), dtype=torch.float32, device=dev)
+            self.wsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)  # forward -> backward
+        else:
+            self.wsel = None
+        if want_count:
+            self.max_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
+            self.min_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
+        query = lib.mam_fc_forward_values_workspace if values_only else lib.mam_fc_forward_workspace
+        self.ws_bytes = query(N, K, M)
+        self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
+        self.sp = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    @staticmethod
+    def _p(t):
+        return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+    def forward(self):
+        P, N, K, M = self._p, self.N, self.K, self.M
+        if self.values_only:
+            rc = self.lib.mam_fc_forward_values(P(self.x), K, P(self.w), K, self.capi.W_MK, None, P(self.c),
+                                                N, K, M, P(self.ws), self.ws_bytes, self.sp)
+        else:
+            rc = self.lib.mam_fc_forward(P(self.x), K, P(self.w), K, self.capi.W_MK, None, P(self.c),
+                                         P(self.amax), P(self.amin), P(self.wsel), N, K, M, P(self.ws),
+                                         self.ws_bytes, self.sp)
+        assert rc == 0, self.lib.mam_last_error()
+
+    def backward(self):
+        P, N, K, M = self._p, self.N, self.K, self.M
+        rc = self.lib.mam_fc_backward(P(self.x), K, P(self.w), K, self.capi.W_MK, P(self.g), P(self.amax),
+                                      P(self.amin), P(self.wsel), P(self.xg), P(self.wg), N, K, M, self.sp)
+        assert rc == 0, self.lib.mam_last_error()
+
+    def count(self):
+        P = self._p
+        rc = self.lib.mam_selection_count(P(self.amax), P(self.amin), P(self.max_count), P(self.min_count),
+                                          self.N, self.M, self.K, self.capi.COUNT_HITS, self.sp)
+        assert rc == 0, self.lib.mam_last_error()
+
+    def backward_bytes(self):
+        N, K, M = self.N, self.K, self.M
+        return 4 * (N * K + N * M + 2 * N * M + 2 * N * M + N * K + K * M)
+
+
+def dense_cpu_baseline(torch, layers_cpu, budget_s, with_backward):
+    """Times the pure-PyTorch port on the first `rows` batch rows of every layer."""
     from oracle import torch_port
 
-    b = w.T.contiguous()
-    rows = 2
-    t0 = time.perf_counter()
-    y, amax, amin = torch_port.forward(x[:rows], b)
-    torch_port.backward(x[:rows], b, g[:rows], amax, amin)
-    per_row = (time.perf_counter() - t0) / rows
-    rows = int(max(2, min(N, budget_s / max(per_row, 1e-6))))
-    t0 = time.perf_counter()
-    y, amax, amin = torch_port.forward(x[:rows], b)
-    torch_port.backward(x[:rows], b, g[:rows], amax, amin)
-    dt = time.perf_counter() - t0
+    def run(rows):
+        t0 = time.perf_counter()
+        for x, w, g in layers_cpu:
+            b = w.T.contiguous()
+            _, amax, amin = torch_port.forward(x[:rows], b)
+            if with_backward:
+                torch_port.backward(x[:rows], b, g[:rows], amax, amin)
+        return time.perf_counter() - t0
+
+    n_rows = layers_cpu[0][0].shape[0]
+    per_row = run(2) / 2
+    rows = int(max(2, min(n_rows, budget_s / max(per_row, 1e-6))))
+    dt = run(rows)
+    triples = sum(rows * x.shape[1] * w.shape[0] for x, w, _ in layers_cpu)
     return {
-        "value": round(rows * K * M / dt / 1e9, 4),
+        "value": round(triples / dt / 1e9, 4),
         "unit": "GOPS",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": "forward+backward of oracle/torch_port.py on the first %d of %d batch rows "
-                  "(%.1f s); rows are independent, so GOPS does not depend on the row count" % (rows, N, dt),
+        "sample": "forward%s of oracle/torch_port.py on the first %d of %d batch rows (%.1f s); rows are "
+                  "independent, so GOPS does not depend on the row count"
+                  % ("+backward" if with_backward else "", rows, n_rows, dt),
     }
+
+
+def time_phases(torch, stream, phases, steps, warmup):
+    """Runs every phase once per step; returns (ms per step by the host clock, ms per phase by events)."""
+    for _ in range(warmup):
+        for _, fn in phases:
+            fn()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(phases) + 1)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        ev[s][0].record(stream)
+        for i, (_, fn) in enumerate(phases):
+            fn()
+            ev[s][i + 1].record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    per_phase = {}
+    for i, (label, _) in enumerate(phases):
+        ms = sum(e[i].elapsed_time(e[i + 1]) for e in ev) / steps
+        per_phase[label] = per_phase.get(label, 0.0) + ms
+    return (t1 - t0) * 1e3 / steps, per_phase
+
+
+def valu_roofline(kernel, triples, ms):
+    tflops = 3.0 * triples / (ms * 1e-3) / 1e12
+    return {"kernel": kernel, "bound": "valu", "achieved": round(tflops, 3), "peak": VALU_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": round(tflops / VALU_PEAK_TFLOPS, 4),
+            "frac_of_vector_fp32_157.3": round(tflops / VECTOR_FP32_PEAK_TFLOPS, 4), "traffic": None}
+
+
+def hbm_roofline(kernel, nbytes, ms):
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": nbytes}
+
+
+def run_dense(torch, capi, lib, dev, args):
+    """headline, values_headline, vit_mlp and inference_*: dense layers in (out, in) weight layout."""
+    gen = torch.Generator().manual_seed(0)
+    wl = args.workload
+    if wl in ("headline", "values_headline"):
+        N, K, M = 256, 4096, 4096
+        x = torch.randn(N, K, generator=gen)
+        w = (torch.rand(M, K, generator=gen) * 2 - 1) / 64.0       # U(-1/64, 1/64)
+        g = torch.randn(N, M, generator=gen)
+        shapes = [(x, w, g)]
+        backward, count, values = wl == "headline", wl == "headline", wl == "values_headline"
+        text = ("MAM FullyConnected fp32 batch 256 in 4096 out 4096: exact forward with argmax/argmin + "
+                "backward (grad_x, grad_W) + selection-count accumulation; x~N(0,1), W~U(-1/64,1/64), "
+                "grad_out~N(0,1), seed 0; weight in (out,in) layout") if wl == "headline" else \
+               "MAM FullyConnected fp32 batch 256 in 4096 out 4096: values-only forward; x~N(0,1), W~U(-1/64,1/64)"
+    elif wl == "vit_mlp":
+        N = 12608
+        shapes = []
+        for K, M in ((768, 3072), (3072, 768)):
+            x = torch.randn(N, K, generator=gen)
+            w = (torch.rand(M, K, generator=gen) * 2 - 1) / K ** 0.5   # Kaiming-uniform(a=sqrt 5)
+            g = torch.randn(N, M, generator=gen)
+            shapes.append((x, w, g))
+        backward, count, values = True, False, False
+        text = ("ViT-B/16-shaped MAM MLP block fp32: 12608 rows, MAM FC 768->3072 then MAM FC 3072->768, each fed "
+                "N(0,1) rows; W Kaiming-uniform; forward + backward of both layers")
+    else:
+        N, K, M = 16384, 4096, int(wl.split("_m")[1])
+        x = torch.rand(N, K, generator=gen) * 2 - 1
+        w = torch.randn(M, K, generator=gen) * 0.02
+        shapes = [(x, w, None)]
+        backward, count, values = False, False, False
+        text = "MAM inference fp32: batch 16384, in 4096, out %d, forward with argmax/argmin; x~U(-1,1), W~N(0,0.02)" % M
+
+    layers = [Layer(torch, capi, lib, dev, x, w, g, backward, count, values) for x, w, g in shapes]
+    phases = []
+    for i, L in enumerate(layers):
+        phases.append(("forward", L.forward))
+    if backward:
+        for L in reversed(layers):
+            phases.append(("backward", L.backward))
+    if count:
+        phases.append(("selection_count", layers[0].count))
+    if wl == "headline":
+        # one plain 64 MiB copy kernel: the known-size reference that scales the profiler's
+        # FETCH_SIZE / WRITE_SIZE counters when traffic is measured
+        calibration_copy = layers[0].max_count.clone()
+        del calibration_copy
+
+    stream = torch.cuda.current_stream(dev)
+    ms_step, ph = time_phases(torch, stream, phases, args.steps, args.warmup)
+    triples = sum(L.N * L.K * L.M for L in layers)
+    fwd_ms = ph["forward"]
+    out = {
+        "config": {"workload": text, "name": wl, "layers": [{"N": L.N, "K": L.K, "M": L.M} for L in layers]},
+        "phases_ms": {k: round(v, 5) for k, v in ph.items()},
+        "forward_gops": round(triples / (fwd_ms * 1e-3) / 1e9, 2),
+    }
+    kernel = "mam_fwd_kernel<MK,%s> + mam_fwd_merge_kernel when K is split (one forward call per layer)" % (
+        "values" if values else "args")
+    out["roofline"] = valu_roofline(kernel, triples, fwd_ms)
+    if wl == "headline":
+        out["roofline"]["traffic"] = sum(FORWARD_TRAFFIC_BYTES.values())
+        out["roofline"]["traffic_by_kernel"] = FORWARD_TRAFFIC_BYTES
+        out["roofline"]["algorithmic_bytes"] = 4 * (256 * 4096 + 4096 * 4096 + 4 * 256 * 4096)
+    if backward:
+        bwd_ms = ph["backward"]
+        out["fwd_bwd_gops"] = round(triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e9, 2)
+        out["fwd_bwd_valu_frac"] = round(3.0 * triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e12 / VALU_PEAK_TFLOPS, 4)
+        out["roofline_backward"] = hbm_roofline("mam_bwd_x_kernel + mam_bwd_w_vec_kernel",
+                                                sum(L.backward_bytes() for L in layers), bwd_ms)
+        if wl == "headline":
+            out["roofline_backward"]["traffic"] = sum(BACKWARD_TRAFFIC_BYTES.values())
+            out["roofline_backward"]["traffic_by_kernel"] = BACKWARD_TRAFFIC_BYTES
+    cpu = None
+    if args.cpu_seconds > 0:
+        cpu = dense_cpu_baseline(torch, shapes, args.cpu_seconds, backward)
+    return triples, ms_step, out, cpu
+
+
+def run_sparse(torch, capi, lib, dev, args):
+    """sparse_d*: CSR forward + backward over a uniformly pruned 4096 x 4096 weight, batch 256."""
+    density = {"sparse_d10": 0.10, "sparse_d03": 0.03, "sparse_d01": 0.01}[args.workload]
+    N, K, M = 256, 4096, 4096
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(N, K, generator=gen)
+    w = torch.randn(M, K, generator=gen) * 0.02
+    g = torch.randn(N, M, generator=gen)
+    keep = max(1, int(round(density * K)))
+    mask = torch.zeros(M, K, dtype=torch.bool)
+    for m in range(M):                                   # seeded random subset of columns per row
+        mask[m, torch.randperm(K, generator=gen)[:keep]] = True
+    dense = w * mask
+    csr = dense.to_sparse_csr()
+    crow, col, val = (t.to(dev) for t in (csr.crow_indices(), csr.col_indices(), csr.values()))
+    nnz = int(val.numel())
+    xd, gd = x.to(dev), g.to(dev)
+    c = torch.empty((N, M), dtype=torch.float32, device=dev)
+    amax = torch.empty((N, M), dtype=torch.int32, device=dev)
+    amin = torch.empty((N, M), dtype=torch.int32, device=dev)
+    xg = torch.empty((N, K), dtype=torch.float32, device=dev)
+    vg = torch.empty((nnz,), dtype=torch.float32, device=dev)
+    ws_bytes = lib.mam_csr_fc_forward_workspace(N, K, M)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    wsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)   # selected values, forward -> backward
+    psel = torch.empty((2, N, M), dtype=torch.int32, device=dev)     # their positions in col/val
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def forward():
+        rc = lib.mam_csr_fc_forward(P(xd), K, P(crow), P(col), P(val), None, P(c), P(amax), P(amin), P(wsel),
+                                    P(psel), N, K, M, nnz, P(ws), ws_bytes, sp)
+        assert rc == 0, lib.mam_last_error()
+
+    def backward():
+        rc = lib.mam_csr_fc_backward(P(xd), K, P(crow), P(col), P(val), P(gd), P(amax), P(amin), P(wsel),
+                                     P(psel), P(xg), P(vg), N, K, M, nnz, sp)
+        assert rc == 0, lib.mam_last_error()
+
+    ms_step, ph = time_phases(torch, stream, [("forward", forward), ("backward", backward)], args.steps, args.warmup)
+    triples = nnz * N                                    # stored products only
+    fwd_bytes = 12 * nnz + 4 * N * K + 12 * N * M + 16 * N * M       # + hand-over arrays
+    bwd_bytes = 4 * N * K + 12 * N * M + 16 * N * M + 4 * N * K + 4 * nnz
+    out = {
+        "config": {"workload": "Pruned CSR-sparse MAM FullyConnected fp32: 4096x4096 weight, %.0f %% of entries kept "
+                               "(seeded random columns per row), W~N(0,0.02), batch 256, x~N(0,1); sparse forward + "
+                               "backward; one op = one stored product" % (density * 100),
+                   "name": args.workload, "N": N, "K": K, "M": M, "nnz": nnz},
+        "phases_ms": {k: round(v, 5) for k, v in ph.items()},
+        "forward_gops": round(triples / (ph["forward"] * 1e-3) / 1e9, 2),
+        "dense_equivalent_forward_gops": round(N * K * M / (ph["forward"] * 1e-3) / 1e9, 2),
+        "roofline": hbm_roofline("transpose_kernel + csr_fwd_kernel", fwd_bytes, ph["forward"]),
+        "roofline_backward": hbm_roofline("mam_bwd_x_kernel + csr_bwd_val_kernel", bwd_bytes, ph["backward"]),
+    }
+    cpu = None
+    if args.cpu_seconds > 0:
+        # dense-equivalent semantics: the port runs on the densified weight; its GOPS are counted in
+        # stored products like `value`
+        cpu = dense_cpu_baseline(torch, [(x, dense, g)], args.cpu_seconds, True)
+        cpu["value"] = round(cpu["value"] * nnz / (K * M), 4)
+        cpu["sample"] += "; densified weight, stored products counted"
+    return triples, ms_step, out, cpu
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=500)
-    ap.add_argument("--warmup", type=int, default=300,
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None,
                     help="untimed steps; the GPU clock needs ~100 launches to ramp up")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
+    ap.add_argument("--workload", choices=WORKLOADS, default="headline")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the MAM hot path has no multi-GPU part in this build "
               "(--gpus %d refused)" % args.gpus, file=sys.stderr)
         sys.exit(2)
+    small = args.workload in ("headline", "values_headline") or args.workload.startswith("sparse")
+    if args.steps is None:
+        args.steps = 500 if small else 20
+    if args.warmup is None:
+        args.warmup = 300 if small else 10
 
     import torch
 
@@ -88,71 +341,8 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     lib = capi.lib()
-    x_cpu, w_cpu, g_cpu = make_inputs(torch, dev)
-    x, w, g = x_cpu.to(dev), w_cpu.to(dev), g_cpu.to(dev)
-
-    c = torch.empty((N, M), dtype=torch.float32, device=dev)
-    amax = torch.empty((N, M), dtype=torch.int32, device=dev)
-    amin = torch.empty((N, M), dtype=torch.int32, device=dev)
-    xg = torch.empty((N, K), dtype=torch.float32, device=dev)
-    wg = torch.empty((M, K), dtype=torch.float32, device=dev)
-    max_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
-    min_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
-    ws_bytes = lib.mam_fc_forward_workspace(N, K, M)
-    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
-    wsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)   # selected weights, forward -> backward
-
-    stream = torch.cuda.current_stream(dev)
-    sp = ctypes.c_void_p(stream.cuda_stream)
-    P = lambda t: ctypes.c_void_p(t.data_ptr())
-
-    def forward():
-        rc = lib.mam_fc_forward(P(x), K, P(w), K, capi.W_MK, None, P(c), P(amax), P(amin), P(wsel),
-                                N, K, M, P(ws), ws_bytes, sp)
-        assert rc == 0, lib.mam_last_error()
-
-    def backward():
-        rc = lib.mam_fc_backward(P(x), K, P(w), K, capi.W_MK, P(g), P(amax), P(amin), P(wsel), P(xg),
-                                 P(wg), N, K, M, sp)
-        assert rc == 0, lib.mam_last_error()
-
-    def count():
-        rc = lib.mam_selection_count(P(amax), P(amin), P(max_count), P(min_count), N, M, K,
-                                     capi.COUNT_HITS, sp)
-        assert rc == 0, lib.mam_last_error()
-
-    # one plain 64 MiB copy kernel: the known-size reference that scales the profiler's
-    # FETCH_SIZE / WRITE_SIZE counters when traffic is measured
-    calibration_copy = max_count.clone()
-    del calibration_copy
-
-    for _ in range(args.warmup):
-        forward(); backward(); count()
-    torch.cuda.synchronize()
-
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for s in range(args.steps):
-        ev[s][0].record(stream)
-        forward()
-        ev[s][1].record(stream)
-        backward()
-        ev[s][2].record(stream)
-        count()
-        ev[s][3].record(stream)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-
-    ms_step = (t1 - t0) * 1e3 / args.steps
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
-    cnt_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
-
-    triples = N * K * M
-    fwd_tflops = 3.0 * triples / (fwd_ms * 1e-3) / 1e12
-    bwd_bytes = 4 * (N * K + N * M + 2 * N * M + 2 * N * M + N * K + K * M)
-    bwd_gbs = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    run = run_sparse if args.workload.startswith("sparse") else run_dense
+    triples, ms_step, extra, cpu = run(torch, capi, lib, dev, args)
 
     out = {
         "metric": "MAM FC fwd+bwd GOPS @4096x4096 b256 fp32; % FP32 VALU peak; bwd HBM GB/s",
@@ -167,45 +357,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {
-            "workload": "MAM FullyConnected fp32 batch 256 in 4096 out 4096: exact forward with "
-                        "argmax/argmin + backward (grad_x, grad_W) + selection-count accumulation; "
-                        "x~N(0,1), W~U(-1/64,1/64), grad_out~N(0,1), seed 0; weight in (out,in) layout",
-            "N": N, "K": K, "M": M,
-        },
-        "phases_ms": {"forward": round(fwd_ms, 5), "backward": round(bwd_ms, 5),
-                      "selection_count": round(cnt_ms, 5)},
-        "forward_gops": round(triples / (fwd_ms * 1e-3) / 1e9, 2),
-        "fwd_bwd_gops": round(triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e9, 2),
-        "fwd_bwd_valu_frac": round(3.0 * triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e12 / VALU_PEAK_TFLOPS, 4),
-        "roofline": {
-            "kernel": "mam_fwd_kernel<MK,args> + mam_fwd_merge_kernel (one mam_fc_forward call)",
-            "bound": "valu",
-            "achieved": round(fwd_tflops, 3),
-            "peak": VALU_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": round(fwd_tflops / VALU_PEAK_TFLOPS, 4),
-            "frac_of_vector_fp32_157.3": round(fwd_tflops / VECTOR_FP32_PEAK_TFLOPS, 4),
-            "traffic": sum(FORWARD_TRAFFIC_BYTES.values()),
-            "traffic_by_kernel": FORWARD_TRAFFIC_BYTES,
-            "algorithmic_bytes": 4 * (N * K + K * M + 4 * N * M),
-        },
-        "roofline_backward": {
-            "kernel": "mam_bwd_x_kernel + mam_bwd_w_vec_kernel",
-            "bound": "hbm",
-            "achieved": round(bwd_gbs, 1),
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(bwd_gbs / HBM_PEAK_GBS, 4),
-            "traffic": sum(BACKWARD_TRAFFIC_BYTES.values()),
-            "traffic_by_kernel": BACKWARD_TRAFFIC_BYTES,
-            "algorithmic_bytes": bwd_bytes,
-        },
     }
-    if args.cpu_seconds > 0:
-        out["cpu_baseline"] = cpu_baseline(torch, x_cpu, w_cpu, g_cpu, args.cpu_seconds)
-    else:
-        out["cpu_baseline"] = None
+    out.update(extra)
+    out["cpu_baseline"] = cpu
     print(json.dumps(out))
 
 

@@ -105,22 +105,29 @@ int mam_selection_count(const int32_t *argmax, const int32_t *argmin, int32_t *m
  * (mamtorch/sparse/kernel/v1/csrc/cuda/cusparsemm_csr.cu:25-45).  The result equals
  * mam_fc_forward on the densified weight: absent entries are zeros that take part in the
  * max/min and in the first-index tie-break.  The reference has no sparse MAM operator.
+ * `workspace` (mam_csr_fc_forward_workspace() bytes, 16-byte aligned) receives x transposed.
+ * `w_sel` and `pos_sel` (optional, may be NULL): (2, N, M) fp32 / int32 contiguous; receive, for the
+ * argmax in plane 0 and the argmin in plane 1, the selected stored value and its position in
+ * col/val (0.0f and -1 where an implicit zero was selected).  Handing both to mam_csr_fc_backward
+ * spares that call a binary search per selection and all atomics in global memory.
  */
 size_t mam_csr_fc_forward_workspace(int64_t N, int64_t K, int64_t M);
 int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                        const float *val, const float *bias, float *c, int32_t *argmax,
-                       int32_t *argmin, int64_t N, int64_t K, int64_t M,
-                       void *workspace, size_t workspace_bytes, void *stream);
+                       int32_t *argmin, float *w_sel, int32_t *pos_sel, int64_t N, int64_t K,
+                       int64_t M, int64_t nnz, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
- * CSR-sparse MAM backward: x_grad (N,K) dense and val_grad (nnz), both fully overwritten.
- * A selected column that is not stored in its row (an implicit zero won) has no weight
- * gradient and adds nothing to x_grad.
+ * CSR-sparse MAM backward: x_grad (N,K) dense and val_grad (nnz), both fully overwritten; either may
+ * be NULL to skip it.  A selected column that is not stored in its row (an implicit zero won) has no
+ * weight gradient and adds nothing to x_grad.  `w_sel` / `pos_sel` (optional, both or neither) are the
+ * arrays written by mam_csr_fc_forward for the same inputs.
  */
 int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                         const float *val, const float *grad, const int32_t *argmax,
-                        const int32_t *argmin, float *x_grad, float *val_grad,
-                        int64_t N, int64_t K, int64_t M, int64_t nnz, void *stream);
+                        const int32_t *argmin, const float *w_sel, const int32_t *pos_sel,
+                        float *x_grad, float *val_grad, int64_t N, int64_t K, int64_t M,
+                        int64_t nnz, void *stream);
 
 #ifdef __cplusplus
 }

@@ -49,10 +49,10 @@ def lib():
         l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
                                       _i64, _i64, _ptr]
         l.mam_selection_count.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr]
-        l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
-                                         _i64, _ptr, _size, _ptr]
-        l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
-                                          _i64, _i64, _i64, _ptr]
+        l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                         _i64, _i64, _i64, _i64, _ptr, _size, _ptr]
+        l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                          _ptr, _i64, _i64, _i64, _i64, _ptr]
         _configured = True
     return l
 
@@ -141,19 +141,23 @@ def selection_count(argmax, argmin, max_count, min_count, mode=COUNT_REFERENCE):
                                      _stream(argmax)))
 
 
-def csr_fc_forward(x, crow, col, val, M, bias=None):
+def csr_fc_forward(x, crow, col, val, M, bias=None, w_sel=None, pos_sel=None):
+    """Returns (c, argmax, argmin); fills the optional (2,N,M) hand-over arrays for the backward."""
     l = lib()
     N, K = x.shape
     c = torch.empty((N, M), dtype=torch.float32, device=x.device)
     amax = torch.empty((N, M), dtype=torch.int32, device=x.device)
     amin = torch.empty((N, M), dtype=torch.int32, device=x.device)
+    need = l.mam_csr_fc_forward_workspace(N, K, M)
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         _check(l.mam_csr_fc_forward(_p(x), _ld(x), _p(crow), _p(col), _p(val), _p(bias), _p(c), _p(amax),
-                                    _p(amin), N, K, M, None, 0, _stream(x)))
+                                    _p(amin), _p(w_sel), _p(pos_sel), N, K, M, val.numel(), _p(ws), need,
+                                    _stream(x)))
     return c, amax, amin
 
 
-def csr_fc_backward(x, crow, col, val, grad, argmax, argmin):
+def csr_fc_backward(x, crow, col, val, grad, argmax, argmin, w_sel=None, pos_sel=None):
     l = lib()
     N, K = x.shape
     M = crow.numel() - 1
@@ -161,5 +165,6 @@ def csr_fc_backward(x, crow, col, val, grad, argmax, argmin):
     vg = torch.empty_like(val)
     with torch.cuda.device(x.device):
         _check(l.mam_csr_fc_backward(_p(x), _ld(x), _p(crow), _p(col), _p(val), _p(grad), _p(argmax),
-                                     _p(argmin), _p(xg), _p(vg), N, K, M, val.numel(), _stream(x)))
+                                     _p(argmin), _p(w_sel), _p(pos_sel), _p(xg), _p(vg), N, K, M, val.numel(),
+                                     _stream(x)))
     return xg, vg

@@ -308,6 +308,18 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
     return rc;
 }
 
+// x_grad from selected weights handed over by a forward, whatever that forward read them from.
+int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t *argmin, const float *w_sel,
+                         float *x_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
+{
+    static const int budget = lds_budget_floats((const void *)mam_bwd_x_kernel<MAM_W_MK>);
+    const int kc = (int)(K < budget ? K : budget);
+    hipLaunchKernelGGL((mam_bwd_x_kernel<MAM_W_MK>), dim3((unsigned)N), dim3(NT_X), (size_t)kc * sizeof(float),
+                       st, (const float *)nullptr, (int64_t)0, grad, argmax, argmin, w_sel, N * M, x_grad, (int)K,
+                       (int)M, kc);
+    return check_launch("mam_bwd_x_kernel");
+}
+
 }  // namespace bwd
 }  // namespace mam
 

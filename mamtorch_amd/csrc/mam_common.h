@@ -38,4 +38,10 @@ __device__ __forceinline__ float load_w(const float *__restrict__ w, int64_t ldw
     return LAYOUT == MAM_W_MK ? w[m * ldw + k] : w[k * ldw + m];
 }
 
+namespace bwd {
+// x_grad (N,K) from the selected weights (2,N,M) written by a forward (mam_backward.hip).
+int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t *argmin, const float *w_sel,
+                         float *x_grad, int64_t N, int64_t K, int64_t M, hipStream_t st);
+}  // namespace bwd
+
 }  // namespace mam

@@ -8,97 +8,219 @@
 // entry is a zero weight whose product x*0 takes part in the max / min and in the first-index
 // tie-break.
 //
-// Forward: a lane owns one CSR row (output neuron) and walks its entries in ascending column
-// order; NB batch rows are register-blocked per lane and their x values are gathered from an LDS
-// copy of the x tile, so HBM sees every (col, val) pair once per batch tile and x once per
-// neuron tile.  While walking, the lane also finds the lowest column missing from its row; the
+// Forward: lanes are batch rows.  x is first transposed into the workspace, xT (K, ldt), so that the
+// x column of a stored entry is contiguous over the batch.  A wave owns one CSR row (output
+// neuron) for a tile of 64*TI batch rows: column indices and values of the row are wave-uniform
+// (scalar loads), each entry costs one coalesced vector load of xT[col], TI multiplies and, per
+// extreme, one strict compare with two selects (value, entry position): the loads bound this
+// kernel, so exact tracking is affordable and nothing is re-scanned afterwards.
+// The lowest column missing from the row is found once per row; the
 // implicit-zero candidate x[n, missing] * 0 is compared last under the dense rule (greater wins,
-// equal -> lower index wins).
+// equal -> lower index wins).  The four waves of a workgroup own four consecutive neurons and
+// hand their results over through LDS so that every batch row stores 16 contiguous bytes.
 //
-// Backward: one workgroup per batch row; selected columns are located in the CSR row by binary
-// search, x_grad is accumulated in an LDS histogram and stored once, val_grad takes global
-// atomic adds (at most N contenders per entry).
+// Backward: when the forward handed over the selected values and their entry positions, x_grad is the
+// dense x_grad kernel fed with those values (an implicit zero contributes 0), and val_grad is
+// accumulated by workgroups that own 8 consecutive CSR rows: an LDS histogram over the rows'
+// entries, streamed out once, no atomics in global memory and no zero fill.  Without the hand-over:
+// one workgroup per batch row; selected columns are located in the CSR row by binary search,
+// x_grad is accumulated in an LDS histogram and stored once, val_grad takes global atomic adds (at
+// most N contenders per entry).
 #include "mam_common.h"
 
 namespace mam {
 namespace csr {
 
 constexpr int NT = 256;
-constexpr int NB = 8;      // batch rows per lane
 constexpr int NT_B = 512;  // backward workgroup
+constexpr int EG = 8;      // entries whose loads are issued together
+constexpr int ROWS = NT / 64;  // CSR rows per forward workgroup (one per wave)
 
-__global__ __launch_bounds__(NT) void csr_fwd_kernel(
-    const float *__restrict__ x, int64_t ldx, const int64_t *__restrict__ crow,
-    const int64_t *__restrict__ col, const float *__restrict__ val, const float *__restrict__ bias,
-    float *__restrict__ c, int32_t *__restrict__ argmax, int32_t *__restrict__ argmin, int N, int K,
-    int M, int kc)
+typedef const __attribute__((address_space(4))) int64_t const_i64;
+typedef const __attribute__((address_space(4))) float const_f32;
+
+// xT[k][n] = x[n][k] for n < N, 0 for N <= n < ldt.  32 x 32 tiles through LDS.
+__global__ __launch_bounds__(256) void transpose_kernel(const float *__restrict__ x, int64_t ldx,
+                                                        float *__restrict__ xT, int ldt, int N, int K)
 {
-    extern __shared__ float xs[];  // [NB][kc]
-    const int tid = threadIdx.x;
-    const int m = blockIdx.x * NT + tid;
-    const int n0 = blockIdx.y * NB;
-    const bool valid = m < M;
-    int64_t e = valid ? crow[m] : 0;
-    const int64_t e_end = valid ? crow[m + 1] : 0;
-    const int64_t row_nnz = e_end - e;
-
-    float vmax[NB], vmin[NB];
-    int imax[NB], imin[NB];
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    const int k0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-        vmax[b] = -__builtin_inff();
-        vmin[b] = __builtin_inff();
-        imax[b] = -1;
-        imin[b] = -1;
+    for (int r = ty; r < 32; r += 8) {
+        const int n = n0 + r, k = k0 + tx;
+        tile[r][tx] = (n < N && k < K) ? x[(int64_t)n * ldx + k] : 0.0f;
     }
-    int missing = 0;  // lowest column not stored in this row (valid once the walk is over)
+    __syncthreads();
+#pragma unroll
+    for (int r = ty; r < 32; r += 8) {
+        const int k = k0 + r, n = n0 + tx;
+        if (k < K && n < ldt) xT[(int64_t)k * ldt + n] = tile[tx][r];
+    }
+}
 
-    for (int k0 = 0; k0 < K; k0 += kc) {
-        const int kn = (K - k0) < kc ? (K - k0) : kc;
+template <int TI> struct XVec;
+template <> struct XVec<1> { typedef float type; };
+template <> struct XVec<4> { typedef float4 type; };
+__device__ __forceinline__ float lane_elem(const float &v, int) { return v; }
+__device__ __forceinline__ float lane_elem(const float4 &v, int t)
+{
+    return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
+}
+
+template <int TI>
+__global__ __launch_bounds__(NT) void csr_fwd_kernel(
+    const float *__restrict__ xT, int ldt, const int64_t *__restrict__ crow,
+    const int64_t *__restrict__ col, const float *__restrict__ val, const float *__restrict__ bias,
+    float *__restrict__ c, int32_t *__restrict__ argmax, int32_t *__restrict__ argmin,
+    float *__restrict__ w_sel, int32_t *__restrict__ pos_sel, int N, int K, int M, int vec_out)
+{
+    typedef typename XVec<TI>::type xvec;
+    constexpr int TILE_N = 64 * TI;
+    __shared__ float out_c[ROWS][TILE_N];
+    __shared__ int out_hi[ROWS][TILE_N], out_lo[ROWS][TILE_N];
+    __shared__ float out_wh[ROWS][TILE_N], out_wl[ROWS][TILE_N];
+    __shared__ int out_ph[ROWS][TILE_N], out_pl[ROWS][TILE_N];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int m = blockIdx.x * ROWS + wave;
+    const int n0 = blockIdx.y * TILE_N;
+    int nl = n0 + lane * TI;
+    if (nl > ldt - TI) nl = ldt - TI;  // lanes past the batch repeat the last rows; never stored
+
+    if (m < M) {
+        const_i64 *ccol = (const_i64 *)col;
+        const_f32 *cval = (const_f32 *)val;
+        const int64_t beg = ((const_i64 *)crow)[m], end = ((const_i64 *)crow)[m + 1];
+        const int nnz = (int)(end - beg);
+        const float *xl = xT + nl;
+
+        // running extremes and the position (within the row) of the entry that set them: strict
+        // compares in ascending entry order, so the first occurrence wins and a zero keeps the sign
+        // of its first occurrence.  The kernel is bound by the xT loads, not by these selects.
+        float vmax[TI], vmin[TI];
+        int pmax[TI], pmin[TI];
 #pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            const int n = (n0 + b) < N ? (n0 + b) : (N - 1);
-            const float *src = x + (int64_t)n * ldx + k0;
-            for (int kk = tid; kk < kn; kk += NT) xs[b * kc + kk] = src[kk];
+        for (int t = 0; t < TI; ++t) {
+            vmax[t] = -__builtin_inff();
+            vmin[t] = __builtin_inff();
+            pmax[t] = -1;
+            pmin[t] = -1;
         }
-        __syncthreads();
-        while (e < e_end) {
-            const int64_t cidx = col[e];
-            if (cidx >= (int64_t)k0 + kn) break;
-            const float v = val[e];
-            const int ci = (int)cidx;
-            if (ci == missing) ++missing;
-            const int kk = ci - k0;
+
+        int i = 0;
+        for (; i + EG <= nnz; i += EG) {
+            xvec xv[EG];
+            float wv[EG];
 #pragma unroll
-            for (int b = 0; b < NB; ++b) {
-                const float p = xs[b * kc + kk] * v;
-                if (p > vmax[b]) { vmax[b] = p; imax[b] = ci; }
-                if (p < vmin[b]) { vmin[b] = p; imin[b] = ci; }
+            for (int u = 0; u < EG; ++u) {
+                xv[u] = *reinterpret_cast<const xvec *>(xl + ccol[beg + i + u] * (int64_t)ldt);
+                wv[u] = cval[beg + i + u];
             }
-            ++e;
-        }
-        __syncthreads();
-    }
-    if (!valid) return;
-
-    const bool has_zero = row_nnz < (int64_t)K;
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-        const int n = n0 + b;
-        if (n >= N) break;
-        float hi = vmax[b], lo = vmin[b];
-        int ih = imax[b], il = imin[b];
-        if (has_zero) {
-            const float z = x[(int64_t)n * ldx + missing] * 0.0f;
-            if (ih < 0 || z > hi || (z == hi && missing < ih)) { hi = z; ih = missing; }
-            if (il < 0 || z < lo || (z == lo && missing < il)) { lo = z; il = missing; }
+            for (int u = 0; u < EG; ++u)
+#pragma unroll
+                for (int t = 0; t < TI; ++t) {
+                    const float pr = lane_elem(xv[u], t) * wv[u];
+                    const bool up = pr > vmax[t], down = pr < vmin[t];
+                    vmax[t] = up ? pr : vmax[t];
+                    pmax[t] = up ? i + u : pmax[t];
+                    vmin[t] = down ? pr : vmin[t];
+                    pmin[t] = down ? i + u : pmin[t];
+                }
         }
-        float s = hi + lo;
-        if (bias) s = s + bias[m];
-        const int64_t o = (int64_t)n * M + m;
-        c[o] = s;
-        argmax[o] = ih;
-        argmin[o] = il;
+        for (; i < nnz; ++i) {
+            const xvec xv = *reinterpret_cast<const xvec *>(xl + ccol[beg + i] * (int64_t)ldt);
+            const float w = cval[beg + i];
+#pragma unroll
+            for (int t = 0; t < TI; ++t) {
+                const float pr = lane_elem(xv, t) * w;
+                const bool up = pr > vmax[t], down = pr < vmin[t];
+                vmax[t] = up ? pr : vmax[t];
+                pmax[t] = up ? i : pmax[t];
+                vmin[t] = down ? pr : vmin[t];
+                pmin[t] = down ? i : pmin[t];
+            }
+        }
+
+        // lowest column missing from the row: stored columns ascend, so it is the first position p
+        // with col[p] != p, or nnz when the row is a full prefix
+        int missing = nnz;
+        for (int base = 0; base < nnz; base += 64) {
+            const int p = base + lane;
+            const bool hole = p < nnz && col[beg + p] != (int64_t)p;
+            const uint64_t mask = __ballot(hole);
+            if (mask) { missing = base + __builtin_ctzll(mask); break; }
+        }
+        const bool has_zero = nnz < K;
+        xvec zx;
+        if (has_zero) zx = *reinterpret_cast<const xvec *>(xl + (int64_t)missing * ldt);
+        const float bm = bias ? bias[m] : 0.0f;
+
+        // column and value of the selected entries (two small divergent loads per extreme)
+        int ri[2][TI];
+        float rw[2][TI];
+#pragma unroll
+        for (int t = 0; t < TI; ++t) {
+            const int e1 = pmax[t] < 0 ? 0 : pmax[t], e2 = pmin[t] < 0 ? 0 : pmin[t];
+            ri[0][t] = (nnz > 0 && pmax[t] >= 0) ? (int)col[beg + e1] : -1;
+            ri[1][t] = (nnz > 0 && pmin[t] >= 0) ? (int)col[beg + e2] : -1;
+            rw[0][t] = (nnz > 0 && pmax[t] >= 0) ? val[beg + e1] : 0.0f;
+            rw[1][t] = (nnz > 0 && pmin[t] >= 0) ? val[beg + e2] : 0.0f;
+        }
+
+#pragma unroll
+        for (int t = 0; t < TI; ++t) {
+            float hi = vmax[t], lo = vmin[t], wh = rw[0][t], wl = rw[1][t];
+            int ih = ri[0][t], il = ri[1][t], ph = pmax[t], pl = pmin[t];
+            if (has_zero) {
+                const float z = lane_elem(zx, t) * 0.0f;
+                if (ih < 0 || z > hi || (z == hi && missing < ih)) { hi = z; ih = missing; wh = 0.0f; ph = -1; }
+                if (il < 0 || z < lo || (z == lo && missing < il)) { lo = z; il = missing; wl = 0.0f; pl = -1; }
+            }
+            float s = hi + lo;
+            if (bias) s = s + bm;
+            const int o = lane * TI + t;
+            out_c[wave][o] = s;
+            out_hi[wave][o] = ih;
+            out_lo[wave][o] = il;
+            out_wh[wave][o] = wh;
+            out_wl[wave][o] = wl;
+            out_ph[wave][o] = ph < 0 ? -1 : (int)(beg + ph);
+            out_pl[wave][o] = pl < 0 ? -1 : (int)(beg + pl);
+        }
+    }
+    __syncthreads();
+
+    // one batch row per thread: ROWS consecutive neurons = 16 contiguous bytes per output array
+    const int m0 = blockIdx.x * ROWS;
+    const int64_t nm = (int64_t)N * M;
+    for (int o = tid; o < TILE_N; o += NT) {
+        const int n = n0 + o;
+        if (n >= N) break;
+        const int64_t base = (int64_t)n * M + m0;
+        if (vec_out && m0 + ROWS <= M) {
+            *reinterpret_cast<float4 *>(c + base) = make_float4(out_c[0][o], out_c[1][o], out_c[2][o], out_c[3][o]);
+            *reinterpret_cast<int4 *>(argmax + base) = make_int4(out_hi[0][o], out_hi[1][o], out_hi[2][o], out_hi[3][o]);
+            *reinterpret_cast<int4 *>(argmin + base) = make_int4(out_lo[0][o], out_lo[1][o], out_lo[2][o], out_lo[3][o]);
+            if (w_sel) {
+                *reinterpret_cast<float4 *>(w_sel + base) = make_float4(out_wh[0][o], out_wh[1][o], out_wh[2][o], out_wh[3][o]);
+                *reinterpret_cast<float4 *>(w_sel + nm + base) = make_float4(out_wl[0][o], out_wl[1][o], out_wl[2][o], out_wl[3][o]);
+            }
+            if (pos_sel) {
+                *reinterpret_cast<int4 *>(pos_sel + base) = make_int4(out_ph[0][o], out_ph[1][o], out_ph[2][o], out_ph[3][o]);
+                *reinterpret_cast<int4 *>(pos_sel + nm + base) = make_int4(out_pl[0][o], out_pl[1][o], out_pl[2][o], out_pl[3][o]);
+            }
+        } else {
+            for (int r = 0; r < ROWS && m0 + r < M; ++r) {
+                c[base + r] = out_c[r][o];
+                argmax[base + r] = out_hi[r][o];
+                argmin[base + r] = out_lo[r][o];
+                if (w_sel) { w_sel[base + r] = out_wh[r][o]; w_sel[nm + base + r] = out_wl[r][o]; }
+                if (pos_sel) { pos_sel[base + r] = out_ph[r][o]; pos_sel[nm + base + r] = out_pl[r][o]; }
+            }
+        }
     }
 }
 
@@ -151,6 +273,77 @@ __global__ __launch_bounds__(NT_B) void csr_bwd_kernel(
     }
 }
 
+constexpr int RB = 8;            // CSR rows per val_grad workgroup
+constexpr int VAL_CAP = 16384;   // histogram floats per pass (64 KiB)
+
+// val_grad of the entries of RB consecutive CSR rows, from the entry positions recorded by the
+// forward (pos_sel, (2, N, M), -1 where an implicit zero was selected).
+__global__ __launch_bounds__(NT) void csr_bwd_val_kernel(
+    const float *__restrict__ x, int64_t ldx, const int64_t *__restrict__ crow,
+    const float *__restrict__ grad, const int32_t *__restrict__ argmax,
+    const int32_t *__restrict__ argmin, const int32_t *__restrict__ pos_sel, int64_t nm,
+    float *__restrict__ val_grad, int N, int M, int vec_in)
+{
+    __shared__ float hist[VAL_CAP];
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.x * RB;
+    const int rows = (M - m0) < RB ? (M - m0) : RB;
+    const int64_t e_beg = crow[m0], e_end = crow[m0 + rows];
+    for (int64_t c0 = e_beg; c0 < e_end; c0 += VAL_CAP) {
+        const int len = (int)((e_end - c0) < VAL_CAP ? (e_end - c0) : VAL_CAP);
+        for (int i = tid; i < len; i += NT) hist[i] = 0.0f;
+        __syncthreads();
+        for (int n = tid; n < N; n += NT) {
+            const int64_t o = (int64_t)n * M + m0;
+            const float *xr = x + (int64_t)n * ldx;
+            float g[RB];
+            int p1[RB], p2[RB], a1[RB], a2[RB];
+            if (vec_in && rows == RB) {
+#pragma unroll
+                for (int q = 0; q < RB / 4; ++q) {
+                    const float4 gv = *reinterpret_cast<const float4 *>(grad + o + 4 * q);
+                    const int4 u1 = *reinterpret_cast<const int4 *>(pos_sel + o + 4 * q);
+                    const int4 u2 = *reinterpret_cast<const int4 *>(pos_sel + nm + o + 4 * q);
+                    const int4 k1 = *reinterpret_cast<const int4 *>(argmax + o + 4 * q);
+                    const int4 k2 = *reinterpret_cast<const int4 *>(argmin + o + 4 * q);
+                    g[4 * q + 0] = gv.x; g[4 * q + 1] = gv.y; g[4 * q + 2] = gv.z; g[4 * q + 3] = gv.w;
+                    p1[4 * q + 0] = u1.x; p1[4 * q + 1] = u1.y; p1[4 * q + 2] = u1.z; p1[4 * q + 3] = u1.w;
+                    p2[4 * q + 0] = u2.x; p2[4 * q + 1] = u2.y; p2[4 * q + 2] = u2.z; p2[4 * q + 3] = u2.w;
+                    a1[4 * q + 0] = k1.x; a1[4 * q + 1] = k1.y; a1[4 * q + 2] = k1.z; a1[4 * q + 3] = k1.w;
+                    a2[4 * q + 0] = k2.x; a2[4 * q + 1] = k2.y; a2[4 * q + 2] = k2.z; a2[4 * q + 3] = k2.w;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < RB; ++r) {
+                    const bool ok = r < rows;
+                    g[r] = ok ? grad[o + r] : 0.0f;
+                    p1[r] = ok ? pos_sel[o + r] : -1;
+                    p2[r] = ok ? pos_sel[nm + o + r] : -1;
+                    a1[r] = ok ? argmax[o + r] : 0;
+                    a2[r] = ok ? argmin[o + r] : 0;
+                }
+            }
+            float x1[RB], x2[RB];
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                const int64_t q1 = (int64_t)p1[r] - c0, q2 = (int64_t)p2[r] - c0;
+                p1[r] = (p1[r] >= 0 && q1 >= 0 && q1 < len) ? (int)q1 : -1;
+                p2[r] = (p2[r] >= 0 && q2 >= 0 && q2 < len) ? (int)q2 : -1;
+                x1[r] = p1[r] >= 0 ? xr[a1[r]] : 0.0f;
+                x2[r] = p2[r] >= 0 ? xr[a2[r]] : 0.0f;
+            }
+#pragma unroll
+            for (int r = 0; r < RB; ++r) {
+                if (p1[r] >= 0) __hip_atomic_fetch_add(&hist[p1[r]], x1[r] * g[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (p2[r] >= 0) __hip_atomic_fetch_add(&hist[p2[r]], x2[r] * g[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+        __syncthreads();
+        for (int i = tid; i < len; i += NT) val_grad[c0 + i] = hist[i];
+        __syncthreads();
+    }
+}
+
 static int lds_budget_floats(const void *kernel)
 {
     constexpr int kWant = 128 * 1024;
@@ -163,51 +356,94 @@ static int lds_budget_floats(const void *kernel)
 }  // namespace csr
 }  // namespace mam
 
-extern "C" size_t mam_csr_fc_forward_workspace(int64_t, int64_t, int64_t) { return 0; }
+static int64_t transposed_ld(int64_t N) { return (N + 3) / 4 * 4; }
+
+extern "C" size_t mam_csr_fc_forward_workspace(int64_t N, int64_t K, int64_t M)
+{
+    if (N <= 0 || K <= 0 || M <= 0) return 0;
+    return (size_t)K * (size_t)transposed_ld(N) * sizeof(float);
+}
 
 extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                                   const float *val, const float *bias, float *c, int32_t *argmax,
-                                  int32_t *argmin, int64_t N, int64_t K, int64_t M, void *workspace,
-                                  size_t workspace_bytes, void *stream)
+                                  int32_t *argmin, float *w_sel, int32_t *pos_sel, int64_t N, int64_t K,
+                                  int64_t M, int64_t nnz, void *workspace, size_t workspace_bytes,
+                                  void *stream)
 {
     using namespace mam;
-    (void)workspace; (void)workspace_bytes;
-    if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
+    if (N < 0 || K < 0 || M < 0 || nnz < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
     if (N == 0 || M == 0) return MAM_OK;
     if (K == 0) return fail(MAM_ERR_INVALID_ARGUMENT, "K == 0: max/min over an empty set");
-    if (!x || !crow || !c || !argmax || !argmin) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    if (!x || !crow || !c || !argmax || !argmin || (nnz > 0 && (!col || !val)))
+        return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
     if (ldx < K) return fail(MAM_ERR_INVALID_ARGUMENT, "ldx smaller than K");
-    if (N > INT32_MAX / 2 || K > INT32_MAX / 2 || M > INT32_MAX / 2)
-        return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
-    static const int budget = csr::lds_budget_floats((const void *)csr::csr_fwd_kernel);
-    int kc = budget / csr::NB;
-    if (K < kc) kc = (int)K;
-    const int64_t gy = ceil_div(N, csr::NB);
-    if (gy > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the CSR forward grid");
-    hipLaunchKernelGGL(csr::csr_fwd_kernel, dim3((unsigned)ceil_div(M, csr::NT), (unsigned)gy),
-                       dim3(csr::NT), (size_t)csr::NB * kc * sizeof(float),
-                       static_cast<hipStream_t>(stream), x, ldx, crow, col, val, bias, c, argmax, argmin,
-                       (int)N, (int)K, (int)M, kc);
+    if (N > INT32_MAX / 2 || K > INT32_MAX / 2 || M > INT32_MAX / 2 || nnz > INT32_MAX)
+        return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30 or nnz exceeds 2^31");
+    const int64_t ldt = transposed_ld(N);
+    const size_t need = (size_t)K * (size_t)ldt * sizeof(float);
+    if (!workspace || workspace_bytes < need || (uintptr_t)workspace % 16 != 0)
+        return fail(MAM_ERR_WORKSPACE, "CSR forward needs %zu workspace bytes, 16-byte aligned, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    float *xT = static_cast<float *>(workspace);
+    const int64_t gk = ceil_div(K, 32), gn = ceil_div(ldt, 32);
+    if (gn > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the transpose grid");
+    hipLaunchKernelGGL(csr::transpose_kernel, dim3((unsigned)gk, (unsigned)gn), dim3(256), 0, st, x, ldx, xT,
+                       (int)ldt, (int)N, (int)K);
+    int rc = check_launch("transpose_kernel");
+    if (rc != MAM_OK) return rc;
+    const int vec_out = (M % 4 == 0) && ((uintptr_t)c % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
+                        ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)w_sel % 16 == 0) &&
+                        ((uintptr_t)pos_sel % 16 == 0);
+    if (N <= 64) {
+        hipLaunchKernelGGL((csr::csr_fwd_kernel<1>), dim3((unsigned)ceil_div(M, csr::ROWS), 1u), dim3(csr::NT), 0,
+                           st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel, pos_sel, (int)N,
+                           (int)K, (int)M, vec_out);
+    } else {
+        const int64_t gy = ceil_div(N, 256);
+        if (gy > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the CSR forward grid");
+        hipLaunchKernelGGL((csr::csr_fwd_kernel<4>), dim3((unsigned)ceil_div(M, csr::ROWS), (unsigned)gy),
+                           dim3(csr::NT), 0, st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel,
+                           pos_sel, (int)N, (int)K, (int)M, vec_out);
+    }
     return check_launch("csr_fwd_kernel");
 }
 
 extern "C" int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                                    const float *val, const float *grad, const int32_t *argmax,
-                                   const int32_t *argmin, float *x_grad, float *val_grad, int64_t N,
-                                   int64_t K, int64_t M, int64_t nnz, void *stream)
+                                   const int32_t *argmin, const float *w_sel, const int32_t *pos_sel,
+                                   float *x_grad, float *val_grad, int64_t N, int64_t K, int64_t M,
+                                   int64_t nnz, void *stream)
 {
     using namespace mam;
     if (N < 0 || K < 0 || M < 0 || nnz < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
     if (N > INT32_MAX / 2 || K > INT32_MAX / 2 || M > INT32_MAX / 2)
         return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool handed = w_sel && pos_sel;
     int rc = MAM_OK;
-    if (val_grad) rc = fill_zero(val_grad, nnz, st);
+    if (val_grad && (!handed || N == 0 || M == 0)) rc = fill_zero(val_grad, nnz, st);
     if (rc != MAM_OK) return rc;
     if (N == 0 || K == 0) return MAM_OK;
     if (M == 0) return x_grad ? fill_zero(x_grad, N * K, st) : MAM_OK;
     if (!x || !crow || !grad || !argmax || !argmin) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
     if (ldx < K) return fail(MAM_ERR_INVALID_ARGUMENT, "ldx smaller than K");
+    if (handed) {
+        if (x_grad) {
+            rc = bwd::x_grad_from_selected(grad, argmax, argmin, w_sel, x_grad, N, K, M, st);
+            if (rc != MAM_OK) return rc;
+        }
+        if (val_grad) {
+            const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
+                               ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)pos_sel % 16 == 0) &&
+                               ((N * M) % 4 == 0);
+            hipLaunchKernelGGL(csr::csr_bwd_val_kernel, dim3((unsigned)ceil_div(M, csr::RB)), dim3(csr::NT), 0, st,
+                               x, ldx, crow, grad, argmax, argmin, pos_sel, N * M, val_grad, (int)N, (int)M,
+                               vec_in);
+            rc = check_launch("csr_bwd_val_kernel");
+        }
+        return rc;
+    }
     static const int budget = csr::lds_budget_floats((const void *)csr::csr_bwd_kernel);
     const int kc = (int)(K < budget ? K : budget);
     hipLaunchKernelGGL(csr::csr_bwd_kernel, dim3((unsigned)N), dim3(csr::NT_B), (size_t)kc * sizeof(float),

@@ -244,7 +244,7 @@ CsrParts csr_parts(const at::Tensor &w_csr, const at::Tensor &a)
     return p;
 }
 
-std::vector<at::Tensor> sparse_fullyconnected(const at::Tensor &a, const at::Tensor &w_csr)
+std::vector<at::Tensor> sparse_forward_impl(const at::Tensor &a, const at::Tensor &w_csr, bool hand_over)
 {
     check_f32_2d(a, "a");
     const CsrParts p = csr_parts(w_csr, a);
@@ -254,18 +254,41 @@ std::vector<at::Tensor> sparse_fullyconnected(const at::Tensor &a, const at::Ten
     auto c = at::empty({N, M}, a.options());
     auto argmax = at::empty({N, M}, a.options().dtype(at::kInt));
     auto argmin = at::empty({N, M}, a.options().dtype(at::kInt));
-    if (N == 0 || M == 0) return {c, argmax, argmin};
-    check_rc(mam_csr_fc_forward(a.data_ptr<float>(), row_stride(a, "a"), p.crow.data_ptr<int64_t>(),
-                                p.col.data_ptr<int64_t>(), p.val.data_ptr<float>(), nullptr,
-                                c.data_ptr<float>(), argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
-                                N, K, M, nullptr, 0, current_stream(a)),
-             "mam_csr_fc_forward");
+    at::Tensor w_sel, pos_sel;
+    if (hand_over) {
+        w_sel = at::empty({2, N, M}, a.options());
+        pos_sel = at::empty({2, N, M}, a.options().dtype(at::kInt));
+    }
+    if (N > 0 && M > 0) {
+        const size_t need = mam_csr_fc_forward_workspace(N, K, M);
+        auto ws = at::empty({(int64_t)(need ? need : 1)}, a.options().dtype(at::kByte));
+        check_rc(mam_csr_fc_forward(a.data_ptr<float>(), row_stride(a, "a"), p.crow.data_ptr<int64_t>(),
+                                    p.col.data_ptr<int64_t>(), p.val.data_ptr<float>(), nullptr,
+                                    c.data_ptr<float>(), argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
+                                    hand_over ? w_sel.data_ptr<float>() : nullptr,
+                                    hand_over ? pos_sel.data_ptr<int32_t>() : nullptr, N, K, M, p.val.numel(),
+                                    ws.data_ptr(), need, current_stream(a)),
+                 "mam_csr_fc_forward");
+    }
+    if (hand_over) return {c, argmax, argmin, w_sel, pos_sel};
     return {c, argmax, argmin};
 }
 
-std::vector<at::Tensor> sparse_fullyconnected_backward(const at::Tensor &a, const at::Tensor &w_csr,
-                                                       const at::Tensor &grad, const at::Tensor &argmax,
-                                                       const at::Tensor &argmin)
+std::vector<at::Tensor> sparse_fullyconnected(const at::Tensor &a, const at::Tensor &w_csr)
+{
+    return sparse_forward_impl(a, w_csr, false);
+}
+
+std::vector<at::Tensor> sparse_fullyconnected_sel(const at::Tensor &a, const at::Tensor &w_csr)
+{
+    return sparse_forward_impl(a, w_csr, true);
+}
+
+std::vector<at::Tensor> sparse_fullyconnected_sel_backward(const at::Tensor &a, const at::Tensor &w_csr,
+                                                           const at::Tensor &grad, const at::Tensor &argmax,
+                                                           const at::Tensor &argmin,
+                                                           const c10::optional<at::Tensor> &w_sel,
+                                                           const c10::optional<at::Tensor> &pos_sel)
 {
     check_f32_2d(a, "a");
     check_f32_2d(grad, "grad");
@@ -274,6 +297,17 @@ std::vector<at::Tensor> sparse_fullyconnected_backward(const at::Tensor &a, cons
     TORCH_CHECK(grad.size(0) == N && grad.size(1) == M, "grad must be (batch, out_features)");
     check_index(argmax, grad, "argmax");
     check_index(argmin, grad, "argmin");
+    const bool handed = w_sel.has_value() && w_sel->defined() && pos_sel.has_value() && pos_sel->defined();
+    if (handed) {
+        TORCH_CHECK(w_sel->scalar_type() == at::kFloat && w_sel->is_contiguous() && w_sel->dim() == 3 &&
+                        w_sel->size(0) == 2 && w_sel->size(1) == N && w_sel->size(2) == M &&
+                        w_sel->device() == a.device(),
+                    "w_sel must be a contiguous float32 (2, batch, out_features) tensor on a's device");
+        TORCH_CHECK(pos_sel->scalar_type() == at::kInt && pos_sel->is_contiguous() && pos_sel->dim() == 3 &&
+                        pos_sel->size(0) == 2 && pos_sel->size(1) == N && pos_sel->size(2) == M &&
+                        pos_sel->device() == a.device(),
+                    "pos_sel must be a contiguous int32 (2, batch, out_features) tensor on a's device");
+    }
     const c10::DeviceGuard guard(a.device());
     const at::Tensor g = grad.contiguous();
     auto a_grad = at::empty({N, K}, a.options());
@@ -281,10 +315,18 @@ std::vector<at::Tensor> sparse_fullyconnected_backward(const at::Tensor &a, cons
     check_rc(mam_csr_fc_backward(a.data_ptr<float>(), row_stride(a, "a"), p.crow.data_ptr<int64_t>(),
                                  p.col.data_ptr<int64_t>(), p.val.data_ptr<float>(), g.data_ptr<float>(),
                                  argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
-                                 a_grad.data_ptr<float>(), val_grad.data_ptr<float>(), N, K, M,
-                                 p.val.numel(), current_stream(a)),
+                                 handed ? w_sel->data_ptr<float>() : nullptr,
+                                 handed ? pos_sel->data_ptr<int32_t>() : nullptr, a_grad.data_ptr<float>(),
+                                 val_grad.data_ptr<float>(), N, K, M, p.val.numel(), current_stream(a)),
              "mam_csr_fc_backward");
     return {a_grad, val_grad};
+}
+
+std::vector<at::Tensor> sparse_fullyconnected_backward(const at::Tensor &a, const at::Tensor &w_csr,
+                                                       const at::Tensor &grad, const at::Tensor &argmax,
+                                                       const at::Tensor &argmin)
+{
+    return sparse_fullyconnected_sel_backward(a, w_csr, grad, argmax, argmin, c10::nullopt, c10::nullopt);
 }
 
 }  // namespace
@@ -310,6 +352,8 @@ TORCH_LIBRARY(mamtorch_kernel_sparsev1, m)
 {
     m.def("fullyconnected(Tensor a, Tensor w_csr) -> Tensor[]");
     m.def("fullyconnected_backward(Tensor a, Tensor w_csr, Tensor grad, Tensor argmax, Tensor argmin) -> Tensor[]");
+    m.def("fullyconnected_sel(Tensor a, Tensor w_csr) -> Tensor[]");
+    m.def("fullyconnected_sel_backward(Tensor a, Tensor w_csr, Tensor grad, Tensor argmax, Tensor argmin, Tensor? w_sel, Tensor? pos_sel) -> Tensor[]");
 }
 
 // On PyTorch-ROCm the HIP device is served by the CUDA dispatch key.
@@ -337,4 +381,6 @@ TORCH_LIBRARY_IMPL(mamtorch_kernel_sparsev1, SparseCsrCUDA, m)
 {
     m.impl("fullyconnected", &sparse_fullyconnected);
     m.impl("fullyconnected_backward", &sparse_fullyconnected_backward);
+    m.impl("fullyconnected_sel", &sparse_fullyconnected_sel);
+    m.impl("fullyconnected_sel_backward", &sparse_fullyconnected_sel_backward);
 }

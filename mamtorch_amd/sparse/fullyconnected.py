@@ -30,18 +30,20 @@ class SparseFullyConnectedFunction(torch.autograd.Function):
     def forward(ctx, a, values, crow_indices, col_indices, out_features):
         w_csr = torch.sparse_csr_tensor(crow_indices, col_indices, values.detach(),
                                         size=(out_features, a.size(1)))
-        c, argmax, argmin = K.fullyconnected.default(a.detach(), w_csr)
-        ctx.save_for_backward(a, values, crow_indices, col_indices, argmax, argmin)
+        # the forward hands the selected values and their positions in `values` to the backward
+        c, argmax, argmin, w_sel, pos_sel = K.fullyconnected_sel.default(a.detach(), w_csr)
+        ctx.save_for_backward(a, values, crow_indices, col_indices, argmax, argmin, w_sel, pos_sel)
         ctx.out_features = out_features
         ctx.mark_non_differentiable(argmax, argmin)
         return c, argmax, argmin
 
     @staticmethod
     def backward(ctx, grad, _gmax, _gmin):
-        a, values, crow_indices, col_indices, argmax, argmin = ctx.saved_tensors
+        a, values, crow_indices, col_indices, argmax, argmin, w_sel, pos_sel = ctx.saved_tensors
         w_csr = torch.sparse_csr_tensor(crow_indices, col_indices, values.detach(),
                                         size=(ctx.out_features, a.size(1)))
-        a_grad, v_grad = K.fullyconnected_backward.default(a.detach(), w_csr, grad.contiguous(), argmax, argmin)
+        a_grad, v_grad = K.fullyconnected_sel_backward.default(a.detach(), w_csr, grad.contiguous(), argmax, argmin,
+                                                               w_sel, pos_sel)
         return a_grad, v_grad, None, None, None
 
 

@@ -20,17 +20,44 @@ def _forward_backward(x, dense, crow, col, val, what, bias=None):
     want = oracle.forward(x.numpy(), dense.numpy(), oracle.W_MK, None if bias is None else bias.numpy())
     xd = x.to(dev)
     parts = [t.to(dev) for t in (crow, col, val)]
-    c, amax, amin = capi.csr_fc_forward(xd, *parts, M, None if bias is None else bias.to(dev))
+    w_sel = torch.full((2, N, M), 7.0, dtype=torch.float32, device=dev)
+    pos_sel = torch.full((2, N, M), -7, dtype=torch.int32, device=dev)
+    c, amax, amin = capi.csr_fc_forward(xd, *parts, M, None if bias is None else bias.to(dev), w_sel, pos_sel)
+    c2, amax2, amin2 = capi.csr_fc_forward(xd, *parts, M, None if bias is None else bias.to(dev))
     torch.cuda.synchronize()
     assert_bits_equal(c.cpu().numpy(), want[0], what + " c")
     assert_index_equal(amax.cpu().numpy(), want[1], what + " argmax")
     assert_index_equal(amin.cpu().numpy(), want[2], what + " argmin")
+    assert torch.equal(c.view(torch.int32), c2.view(torch.int32)) and torch.equal(amax, amax2) and torch.equal(amin, amin2)
+    # hand-over arrays: position of the selected entry in col/val (-1: an implicit zero) and its value
+    pos = pos_sel.cpu().numpy().astype(np.int64)
+    sel = np.stack([want[1], want[2]]).astype(np.int64)
+    rows_of = np.broadcast_to(np.arange(M), (2, N, M))
+    stored = pos >= 0
+    assert (pos[stored] >= crow.numpy()[rows_of[stored]]).all() and (pos[stored] < crow.numpy()[rows_of[stored] + 1]).all()
+    assert (col.numpy()[pos[stored]] == sel[stored]).all(), what + " pos_sel points at another column"
+    assert (dense.numpy()[rows_of[~stored], sel[~stored]] == 0).all()
+    is_stored = np.zeros((M, K), dtype=bool)
+    is_stored[np.repeat(np.arange(M), np.diff(crow.numpy())), col.numpy()] = True
+    assert (is_stored[rows_of, sel] == stored).all(), what + " pos_sel misses a stored column"
+    ws = w_sel.cpu().numpy()
+    assert_bits_equal(ws[stored], val.numpy()[pos[stored]], what + " w_sel")
+    assert (ws[~stored] == 0).all()
     grad = torch.randn(N, M, generator=torch.Generator().manual_seed(1))
     xo, vo = oracle.csr_backward(x.numpy(), crow.numpy(), col.numpy(), val.numpy(), grad.numpy(), want[1], want[2])
-    xg, vg = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin)
-    torch.cuda.synchronize()
-    np.testing.assert_allclose(xg.cpu().numpy(), xo, rtol=1e-5, atol=1e-6, err_msg=what + " x_grad")
-    np.testing.assert_allclose(vg.cpu().numpy(), vo, rtol=1e-5, atol=1e-6, err_msg=what + " val_grad")
+    # rtol 1e-5 plus the rounding floor of an fp32 sum in any order: 2^-22 x the sum of |terms| of the
+    # cell, measured by the oracle's backward over absolute values
+    xa, va = oracle.csr_backward(np.abs(x.numpy()), crow.numpy(), col.numpy(), np.abs(val.numpy()),
+                                 np.abs(grad.numpy()), want[1], want[2])
+    for handed in (False, True):
+        xg, vg = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin,
+                                      w_sel if handed else None, pos_sel if handed else None)
+        torch.cuda.synchronize()
+        tag = what + (" (hand-over)" if handed else " (search)")
+        for got, wanted, floor, name in ((xg, xo, xa, "x_grad"), (vg, vo, va, "val_grad")):
+            err = np.abs(got.cpu().numpy().astype(np.float64) - wanted)
+            bound = 1e-5 * np.abs(wanted) + 2.0 ** -22 * floor + 1e-30
+            assert (err <= bound).all(), "%s %s: worst excess %g" % (tag, name, (err - bound).max())
     # stored positions agree with the dense backward; pruned positions get nothing
     xdense, wdense = oracle.backward(x.numpy(), dense.numpy(), grad.numpy(), want[1], want[2], oracle.W_MK)
     np.testing.assert_allclose(xo, xdense, rtol=1e-6, atol=1e-7)
@@ -44,6 +71,15 @@ def test_densities(density):
     dense, crow, col, val = pruned_csr(M, K, density, seed=int(density * 100))
     x = torch.randn(N, K, generator=torch.Generator().manual_seed(2))
     _forward_backward(x, dense, crow, col, val, "density %g" % density)
+
+
+@pytest.mark.parametrize("N,M,K", [(301, 130, 257), (64, 7, 33), (65, 9, 4), (1, 5, 300), (517, 66, 100)])
+def test_batch_tiles_and_ragged_shapes(N, M, K):
+    # more than one batch tile, batch sizes that are no multiple of 4, neuron counts that are no
+    # multiple of the 4 rows of a workgroup, unaligned row lengths
+    dense, crow, col, val = pruned_csr(M, K, 0.2, seed=N + M)
+    x = torch.randn(N, K, generator=torch.Generator().manual_seed(N))
+    _forward_backward(x, dense, crow, col, val, "N%d M%d K%d" % (N, M, K))
 
 
 def test_implicit_zero_rules():
@@ -108,7 +144,12 @@ def test_config5_full_size_equals_dense_kernel(density):
     assert_bits_equal(c[rows.to(dev)].cpu().numpy(), want[0], "config 5 c")
     assert_index_equal(amax[rows.to(dev)].cpu().numpy(), want[1], "config 5 argmax")
     grad = torch.randn(N, M, generator=torch.Generator().manual_seed(6))
+    w_sel = torch.empty((2, N, M), dtype=torch.float32, device=dev)
+    pos_sel = torch.empty((2, N, M), dtype=torch.int32, device=dev)
+    c3, amax3, amin3 = capi.csr_fc_forward(xd, *parts, M, None, w_sel, pos_sel)
+    assert torch.equal(c3.view(torch.int32), cd.view(torch.int32)) and torch.equal(amax3, dmax)
     xg, vg = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin)
+    xg2, vg2 = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin, w_sel, pos_sel)
     xdg, wdg = capi.fc_backward(xd, dense.to(dev), grad.to(dev), amax, amin, capi.W_MK)
     torch.cuda.synchronize()
     # two fp32 summation orders of the same terms: each may be off by the rounding floor of the
@@ -117,5 +158,6 @@ def test_config5_full_size_equals_dense_kernel(density):
     torch.cuda.synchronize()
     rws = torch.repeat_interleave(torch.arange(M), crow[1:] - crow[:-1]).to(dev)
     want_v, abs_v = wdg[rws, col.to(dev)], wabs[rws, col.to(dev)]
-    assert bool(((xg - xdg).abs() <= 1e-5 * xdg.abs() + 2.0 ** -21 * xabs).all())
-    assert bool(((vg - want_v).abs() <= 1e-5 * want_v.abs() + 2.0 ** -21 * abs_v).all())
+    for got_x, got_v in ((xg, vg), (xg2, vg2)):
+        assert bool(((got_x - xdg).abs() <= 1e-5 * xdg.abs() + 2.0 ** -21 * xabs).all())
+        assert bool(((got_v - want_v).abs() <= 1e-5 * want_v.abs() + 2.0 ** -21 * abs_v).all())
