@@ -109,15 +109,19 @@ __global__ __launch_bounds__(NT) void csr_fwd_kernel(
             pmin[t] = -1;
         }
 
-        int i = 0;
-        for (; i + EG <= nnz; i += EG) {
-            xvec xv[EG];
-            float wv[EG];
+        // full groups of EG entries, software-pipelined: the loads of group g+1 are in flight while
+        // group g is consumed, so a row costs about one memory round trip per group
+        const int ng = nnz / EG;
+        xvec xa[EG], xb[EG];
+        float wa[EG], wb[EG];
+        auto issue = [&](int g, xvec (&xv)[EG], float (&wv)[EG]) {
 #pragma unroll
             for (int u = 0; u < EG; ++u) {
-                xv[u] = *reinterpret_cast<const xvec *>(xl + ccol[beg + i + u] * (int64_t)ldt);
-                wv[u] = cval[beg + i + u];
+                xv[u] = *reinterpret_cast<const xvec *>(xl + ccol[beg + g * EG + u] * (int64_t)ldt);
+                wv[u] = cval[beg + g * EG + u];
             }
+        };
+        auto consume = [&](int g, const xvec (&xv)[EG], const float (&wv)[EG]) {
 #pragma unroll
             for (int u = 0; u < EG; ++u)
 #pragma unroll
@@ -125,11 +129,26 @@ __global__ __launch_bounds__(NT) void csr_fwd_kernel(
                     const float pr = lane_elem(xv[u], t) * wv[u];
                     const bool up = pr > vmax[t], down = pr < vmin[t];
                     vmax[t] = up ? pr : vmax[t];
-                    pmax[t] = up ? i + u : pmax[t];
+                    pmax[t] = up ? g * EG + u : pmax[t];
                     vmin[t] = down ? pr : vmin[t];
-                    pmin[t] = down ? i + u : pmin[t];
+                    pmin[t] = down ? g * EG + u : pmin[t];
                 }
+        };
+        // two register buffers, the loop unrolled by two groups, so that no copy (which would
+        // have to wait for the data) sits between issuing and consuming
+        if (ng > 0) issue(0, xa, wa);
+        for (int g = 0; g < ng; g += 2) {
+            if (g + 1 < ng) issue(g + 1, xb, wb);
+            __builtin_amdgcn_sched_barrier(0);
+            consume(g, xa, wa);
+            __builtin_amdgcn_sched_barrier(0);
+            if (g + 1 >= ng) break;
+            if (g + 2 < ng) issue(g + 2, xa, wa);
+            __builtin_amdgcn_sched_barrier(0);
+            consume(g + 1, xb, wb);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        int i = ng * EG;
         for (; i < nnz; ++i) {
             const xvec xv = *reinterpret_cast<const xvec *>(xl + ccol[beg + i] * (int64_t)ldt);
             const float w = cval[beg + i];
