@@ -19,6 +19,8 @@ Other workloads (`--workload`), same JSON layout, used for the tables in the des
   inference_m{1024,4096,16384}   batch 16384, in 4096, forward with indices only
   values_headline    headline shape, values-only forward
   sparse_d{10,03,01} 4096x4096 weight pruned to 10 % / 3 % / 1 %, batch 256, CSR forward + backward
+  spmm_d{30,10,01}   sum-of-products SpMM (cusparsemm): 4096x4096 CSR with 30 % / 10 % / 1 % stored, times a
+                     dense 4096x4096; one op = one multiply-add; torch.sparse.mm timed beside it
 """
 import argparse
 import ctypes
@@ -40,7 +42,7 @@ FORWARD_TRAFFIC_BYTES = {"mam_fwd_kernel": 141.1e6, "mam_fwd_merge_kernel": 167.
 BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 103.4e6}
 
 WORKLOADS = ("headline", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
-             "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01")
+             "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01")
 
 
 class Layer:
@@ -313,6 +315,54 @@ def run_sparse(torch, capi, lib, dev, args):
     return triples, ms_step, out, cpu
 
 
+def run_spmm(torch, capi, lib, dev, args):
+    """spmm_d*: c = A @ b, A 4096 x 4096 CSR with Bernoulli-kept N(0,1) entries (the reference's own
+    generator, test/test_sparse.py:14-17), b dense 4096 x 4096."""
+    keep = {"spmm_d30": 0.30, "spmm_d10": 0.10, "spmm_d01": 0.01}[args.workload]
+    R = K = C = 4096
+    gen = torch.Generator().manual_seed(0)
+    a = torch.randn(R, K, generator=gen) * torch.bernoulli(torch.full((R, K), keep), generator=gen)
+    b = torch.randn(K, C, generator=gen)
+    csr = a.to_sparse_csr()
+    crow, col, val = (t.to(dev) for t in (csr.crow_indices(), csr.col_indices(), csr.values()))
+    nnz = int(val.numel())
+    bd = b.to(dev)
+    c = torch.empty((R, C), dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def spmm():
+        rc = lib.mam_csr_spmm(P(crow), P(col), P(val), P(bd), C, P(c), R, K, C, sp)
+        assert rc == 0, lib.mam_last_error()
+
+    ms_step, ph = time_phases(torch, stream, [("spmm", spmm)], args.steps, args.warmup)
+    csr_dev = torch.sparse_csr_tensor(crow, col, val, size=(R, K))
+    _, ph_lib = time_phases(torch, stream, [("torch.sparse.mm", lambda: torch.sparse.mm(csr_dev, bd))],
+                            max(args.steps // 10, 5), 5)
+    ops = nnz * C
+    nbytes = 12 * nnz + 4 * K * C + 4 * R * C
+    out = {
+        "config": {"workload": "sum-of-products SpMM fp32: A 4096x4096 CSR, %.0f %% of entries stored (Bernoulli mask "
+                               "on N(0,1), seed 0), times dense b 4096x4096; one op = one multiply-add"
+                               % (keep * 100), "name": args.workload, "R": R, "K": K, "C": C, "nnz": nnz},
+        "phases_ms": {k: round(v, 5) for k, v in ph.items()},
+        "library_ms": {k: round(v, 5) for k, v in ph_lib.items()},
+        "operand_fetch_tbs": round(4.0 * nnz * C / (ph["spmm"] * 1e-3) / 1e12, 2),
+        "roofline": hbm_roofline("csr_spmm_kernel", nbytes, ph["spmm"]),
+    }
+    cpu = None
+    if args.cpu_seconds > 0:
+        rows = 256
+        t0 = time.perf_counter()
+        torch.sparse.mm(a[:rows].to_sparse_csr(), b)
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(int((a[:rows] != 0).sum()) * C / dt / 1e9, 4), "unit": "GOPS",
+               "cores": torch.get_num_threads(), "kind": "port",
+               "sample": "torch.sparse.mm on the CPU over the first %d rows of A (%.2f s)" % (rows, dt)}
+    return ops, ms_step, out, cpu
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -327,6 +377,9 @@ def main():
               "(--gpus %d refused)" % args.gpus, file=sys.stderr)
         sys.exit(2)
     small = args.workload in ("headline", "values_headline") or args.workload.startswith("sparse")
+    if args.workload.startswith("spmm"):
+        args.steps = 50 if args.steps is None else args.steps
+        args.warmup = 20 if args.warmup is None else args.warmup
     if args.steps is None:
         args.steps = 500 if small else 20
     if args.warmup is None:
@@ -341,7 +394,8 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     lib = capi.lib()
-    run = run_sparse if args.workload.startswith("sparse") else run_dense
+    run = run_sparse if args.workload.startswith("sparse") else run_spmm if args.workload.startswith("spmm") \
+        else run_dense
     triples, ms_step, extra, cpu = run(torch, capi, lib, dev, args)
 
     out = {

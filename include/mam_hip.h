@@ -129,6 +129,21 @@ int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *crow, const 
                         float *x_grad, float *val_grad, int64_t N, int64_t K, int64_t M,
                         int64_t nnz, void *stream);
 
+/*
+ * Sum-of-products SpMM: c (R, C) contiguous = A (R, K) sparse @ b (K, C) dense with row stride ldb,
+ * fp32, alpha 1, beta 0.  Replace mamtorch_kernel_sparsev1::cusparsemm_csr
+ * (mamtorch/sparse/kernel/v1/csrc/cuda/cusparsemm_csr.cu:19-77) and ::cusparsemm_coo
+ * (mamtorch/sparse/kernel/v1/csrc/cuda/cusparsemm_coo.cu:19-76), both thin wrappers of cusparseSpMM with
+ * int64 indices.  CSR: crow (R+1), col / val (nnz); any column order within a row.  COO: row / col / val
+ * (nnz) in any order, repeated coordinates add up (as an uncoalesced torch COO tensor means); c is
+ * accumulated with atomic adds, so its rounding can differ from run to run when a row spans more than
+ * 64 consecutive entries.
+ */
+int mam_csr_spmm(const int64_t *crow, const int64_t *col, const float *val, const float *b, int64_t ldb,
+                 float *c, int64_t R, int64_t K, int64_t C, void *stream);
+int mam_coo_spmm(const int64_t *row, const int64_t *col, const float *val, int64_t nnz, const float *b,
+                 int64_t ldb, float *c, int64_t R, int64_t K, int64_t C, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -21,6 +21,7 @@ EXPORTS = (
     "mam_fc_forward_values_workspace", "mam_fc_forward_values",
     "mam_fc_backward", "mam_selection_count",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward",
+    "mam_csr_spmm", "mam_coo_spmm",
 )
 
 _i64 = ctypes.c_int64
@@ -53,6 +54,8 @@ def lib():
                                          _i64, _i64, _i64, _i64, _ptr, _size, _ptr]
         l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                           _ptr, _i64, _i64, _i64, _i64, _ptr]
+        l.mam_csr_spmm.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
+        l.mam_coo_spmm.argtypes = [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
         _configured = True
     return l
 
@@ -168,3 +171,23 @@ def csr_fc_backward(x, crow, col, val, grad, argmax, argmin, w_sel=None, pos_sel
                                      _p(argmin), _p(w_sel), _p(pos_sel), _p(xg), _p(vg), N, K, M, val.numel(),
                                      _stream(x)))
     return xg, vg
+
+
+def csr_spmm(crow, col, val, b, R):
+    """c (R, C) = A (R, K) in CSR @ b (K, C) dense (rows may be strided)."""
+    l = lib()
+    K, C = b.shape
+    c = torch.empty((R, C), dtype=torch.float32, device=b.device)
+    with torch.cuda.device(b.device):
+        _check(l.mam_csr_spmm(_p(crow), _p(col), _p(val), _p(b), _ld(b), _p(c), R, K, C, _stream(b)))
+    return c
+
+
+def coo_spmm(row, col, val, b, R):
+    """c (R, C) = A (R, K) in COO (any order, duplicates add up) @ b (K, C) dense."""
+    l = lib()
+    K, C = b.shape
+    c = torch.empty((R, C), dtype=torch.float32, device=b.device)
+    with torch.cuda.device(b.device):
+        _check(l.mam_coo_spmm(_p(row), _p(col), _p(val), val.numel(), _p(b), _ld(b), _p(c), R, K, C, _stream(b)))
+    return c

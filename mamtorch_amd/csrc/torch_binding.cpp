@@ -329,6 +329,53 @@ std::vector<at::Tensor> sparse_fullyconnected_backward(const at::Tensor &a, cons
     return sparse_fullyconnected_sel_backward(a, w_csr, grad, argmax, argmin, c10::nullopt, c10::nullopt);
 }
 
+// ---- sum-of-products SpMM: a sparse (R, K), b dense (K, C) -> dense (R, C) ----
+// Schema and keys of mamtorch/sparse/kernel/v1/csrc/cuda/register_functions.cu:18-28.
+void check_spmm_operands(const at::Tensor &a, const at::Tensor &b)
+{
+    check_f32_2d(b, "b");
+    TORCH_CHECK(a.dim() == 2 && a.size(1) == b.size(0), "a must be (rows, k) with k = b.size(0)");
+    TORCH_CHECK(a.scalar_type() == at::kFloat, "a must be float32");
+    TORCH_CHECK(a.device() == b.device(), "a and b are on different devices");
+}
+
+at::Tensor cusparsemm_csr(const at::Tensor &a, const at::Tensor &b)
+{
+    TORCH_CHECK(a.layout() == at::kSparseCsr, "a must be a torch.sparse_csr tensor");
+    check_spmm_operands(a, b);
+    const int64_t R = a.size(0), K = a.size(1), C = b.size(1);
+    const c10::DeviceGuard guard(b.device());
+    const at::Tensor crow = a.crow_indices().to(at::kLong).contiguous();
+    const at::Tensor col = a.col_indices().to(at::kLong).contiguous();
+    const at::Tensor val = a.values().contiguous();
+    auto c = at::empty({R, C}, b.options());
+    if (R == 0 || C == 0) return c;
+    check_rc(mam_csr_spmm(crow.data_ptr<int64_t>(), col.data_ptr<int64_t>(), val.data_ptr<float>(),
+                          b.data_ptr<float>(), row_stride(b, "b"), c.data_ptr<float>(), R, K, C,
+                          current_stream(b)),
+             "mam_csr_spmm");
+    return c;
+}
+
+at::Tensor cusparsemm_coo(const at::Tensor &a, const at::Tensor &b)
+{
+    TORCH_CHECK(a.layout() == at::kSparse, "a must be a torch.sparse_coo tensor");
+    check_spmm_operands(a, b);
+    TORCH_CHECK(a.sparse_dim() == 2 && a.dense_dim() == 0, "a must have two sparse dimensions");
+    const int64_t R = a.size(0), K = a.size(1), C = b.size(1);
+    const c10::DeviceGuard guard(b.device());
+    const at::Tensor idx = a._indices().to(at::kLong).contiguous();   // (2, nnz); need not be coalesced
+    const at::Tensor val = a._values().contiguous();
+    const int64_t nnz = val.numel();
+    auto c = at::empty({R, C}, b.options());
+    if (R == 0 || C == 0) return c;
+    check_rc(mam_coo_spmm(idx.data_ptr<int64_t>(), idx.data_ptr<int64_t>() + nnz, val.data_ptr<float>(), nnz,
+                          b.data_ptr<float>(), row_stride(b, "b"), c.data_ptr<float>(), R, K, C,
+                          current_stream(b)),
+             "mam_coo_spmm");
+    return c;
+}
+
 }  // namespace
 
 TORCH_LIBRARY(mamtorch_kernel_v1, m)
@@ -352,6 +399,7 @@ TORCH_LIBRARY(mamtorch_kernel_sparsev1, m)
 {
     m.def("fullyconnected(Tensor a, Tensor w_csr) -> Tensor[]");
     m.def("fullyconnected_backward(Tensor a, Tensor w_csr, Tensor grad, Tensor argmax, Tensor argmin) -> Tensor[]");
+    m.def("cusparsemm(Tensor a, Tensor b) -> Tensor");
     m.def("fullyconnected_sel(Tensor a, Tensor w_csr) -> Tensor[]");
     m.def("fullyconnected_sel_backward(Tensor a, Tensor w_csr, Tensor grad, Tensor argmax, Tensor argmin, Tensor? w_sel, Tensor? pos_sel) -> Tensor[]");
 }
@@ -383,4 +431,10 @@ TORCH_LIBRARY_IMPL(mamtorch_kernel_sparsev1, SparseCsrCUDA, m)
     m.impl("fullyconnected_backward", &sparse_fullyconnected_backward);
     m.impl("fullyconnected_sel", &sparse_fullyconnected_sel);
     m.impl("fullyconnected_sel_backward", &sparse_fullyconnected_sel_backward);
+    m.impl("cusparsemm", &cusparsemm_csr);
+}
+
+TORCH_LIBRARY_IMPL(mamtorch_kernel_sparsev1, SparseCUDA, m)
+{
+    m.impl("cusparsemm", &cusparsemm_coo);
 }

@@ -1,10 +1,11 @@
-"""CSR-sparse MAM over pruned weights.
+"""Sparse operators over pruned weights.
 
-The reference's ``mamtorch.sparse`` holds only a cuSPARSE sum-of-products SpMM
-(mamtorch/sparse/kernel/v1/cusparsemm.py:9-10); its CSR operand convention (int64 crow/col,
-fp32 values, sparse operand first in the reference's SpMM, dispatched on the sparse-CSR key) is
-kept for the MAM operators defined here.
+``kernel.v1.cusparsemm`` is the reference's sum-of-products SpMM under its own name
+(mamtorch/sparse/kernel/v1/cusparsemm.py:9-10).  The CSR-sparse MAM operators, which the reference
+does not have, keep that operator's CSR operand convention (int64 crow/col, fp32 values, sparse
+operand dispatched on the sparse-CSR key).
 """
+from . import kernel
 from .fullyconnected import fullyconnected, fullyconnected_backward, SparseFullyConnectedFunction, prune_to_csr
 
-__all__ = ["fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr"]
+__all__ = ["kernel", "fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr"]

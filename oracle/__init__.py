@@ -125,3 +125,24 @@ def csr_backward(x, crow, col, val, grad, argmax, argmin):
     lib().mam_oracle_csr_backward(_p(x), _I64(K), _p(crow), _p(col), _p(val), _p(grad), _p(argmax),
                                   _p(argmin), _p(xg), _p(vg), _I64(N), _I64(K), _I64(M))
     return xg, vg
+
+
+def coo_spmm(row, col, val, b, R):
+    """(c, abs_sum) for c = A @ b with A given as COO triples (any order, duplicates add up); fp64
+    accumulation.  abs_sum[r, j] = sum of |val * b| of the cell: the scale of its rounding floor."""
+    row, col, val = _i64(row), _i64(col), _f32(val)
+    b = _f32(b)
+    K, C = b.shape
+    c = np.empty((R, C), np.float32)
+    ab = np.empty((R, C), np.float32)
+    lib().mam_oracle_coo_spmm(_p(row), _p(col), _p(val), _I64(val.shape[0]), _p(b), _I64(C), _p(c), _p(ab),
+                              _I64(R), _I64(C))
+    return c, ab
+
+
+def csr_spmm(crow, col, val, b):
+    """(c, abs_sum) for c = A @ b with A in CSR (int64 crow / col)."""
+    crow = _i64(crow)
+    R = crow.shape[0] - 1
+    row = np.repeat(np.arange(R, dtype=np.int64), np.diff(crow))
+    return coo_spmm(row, col, val, b, R)

@@ -21,6 +21,14 @@
  *               reference prunes by writing literal zeros into dense weights
  *               (examples/vitb16_imagenet1k/pruning_utils.py:107,111).
  *
+ *   SpMM      : mamtorch/sparse/kernel/v1/csrc/cuda/cusparsemm_csr.cu:19-77 and
+ *               cusparsemm_coo.cu:19-76: C = A_sparse @ B with alpha 1, beta 0 through
+ *               cuSPARSE (third party, absent here; the reference's own test only prints
+ *               the max-abs error against the dense a@b, test/test_sparse.py:33-44).  The
+ *               restatement is the defining sum, accumulated in fp64; it returns the sum of
+ *               |terms| as well, which is what a tolerance for any fp32 summation order
+ *               is made of.  Pinned against numpy's dense matmul and scipy.sparse.
+ *
  * Arithmetic: every product is ONE round-to-nearest fp32 multiply, max+min is one
  * fp32 add, bias one more fp32 add.  Build with -ffp-contract=off.
  *
@@ -177,4 +185,31 @@ void mam_oracle_csr_backward(const float *x, int64_t ldx, const int64_t *crow, c
     for (int64_t i = 0; i < N * K; ++i) x_grad[i] = (float)xa[i];
     for (int64_t i = 0; i < nnz; ++i) val_grad[i] = (float)va[i];
     free(xa); free(va);
+}
+
+/*
+ * SpMM in COO form (a CSR caller expands crow): c (R,C) = sum over entries e of
+ * val[e] * b[col[e], :] added to row row[e]; entries in any order, duplicates add up.
+ * c and, when abs_sum != NULL, the sum of |val*b| per cell are fp64 sums rounded to fp32.
+ */
+void mam_oracle_coo_spmm(const int64_t *row, const int64_t *col, const float *val, int64_t nnz,
+                         const float *b, int64_t ldb, float *c, float *abs_sum, int64_t R, int64_t C)
+{
+    double *acc = (double *)calloc((size_t)(R * C > 0 ? R * C : 1), sizeof(double));
+    double *aab = (double *)calloc((size_t)(R * C > 0 ? R * C : 1), sizeof(double));
+    for (int64_t e = 0; e < nnz; ++e) {
+        const double v = (double)val[e];
+        const float *br = b + col[e] * ldb;
+        double *cr = acc + row[e] * C, *ar = aab + row[e] * C;
+        for (int64_t j = 0; j < C; ++j) {
+            const double t = v * (double)br[j];
+            cr[j] += t;
+            ar[j] += t < 0 ? -t : t;
+        }
+    }
+    for (int64_t i = 0; i < R * C; ++i) {
+        c[i] = (float)acc[i];
+        if (abs_sum) abs_sum[i] = (float)aab[i];
+    }
+    free(acc); free(aab);
 }

@@ -1,0 +1,111 @@
+"""GPU parity of the sum-of-products SpMM (mamtorch_kernel_sparsev1::cusparsemm) through the C ABI and
+through the operator.  The reference checks it by printing the max-abs error against the dense
+``a @ b`` (test/test_sparse.py:33-44); here every cell must be within rtol 1e-5 of the fp64 oracle plus
+the rounding floor of an fp32 sum in any order, 2^-22 x the sum of |terms| of that cell."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def _random_sparse(rows, k, sparse_rate, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(rows, k, generator=g)
+    return a * torch.bernoulli(torch.full((rows, k), 1 - sparse_rate), generator=g)
+
+
+def _check(got, want, floor, what):
+    err = np.abs(got.cpu().numpy().astype(np.float64) - want)
+    bound = 1e-5 * np.abs(want) + 2.0 ** -22 * floor + 1e-30
+    assert (err <= bound).all(), "%s: worst excess %g at %s" % (what, (err - bound).max(),
+                                                                 np.unravel_index((err - bound).argmax(), err.shape))
+
+
+SHAPES = [(37, 53, 29, 0.9), (200, 310, 64, 0.7), (5, 1, 3, 0.0), (64, 64, 100, 0.99), (1, 40, 256, 0.5),
+          (300, 1000, 260, 0.9), (129, 17, 4, 0.2), (33, 90, 1, 0.5), (0, 5, 7, 0.5), (6, 5, 0, 0.5)]
+
+
+@pytest.mark.parametrize("rows,k,cols,rate", SHAPES)
+def test_csr_and_coo_against_oracle(rows, k, cols, rate):
+    from mamtorch_amd import capi
+
+    a = _random_sparse(rows, k, rate, seed=rows + cols)
+    b = torch.randn(k, cols, generator=torch.Generator().manual_seed(k))
+    csr = a.to_sparse_csr()
+    crow, col, val = csr.crow_indices(), csr.col_indices(), csr.values()
+    want, floor = oracle.csr_spmm(crow.numpy(), col.numpy(), val.numpy(), b.numpy())
+    c = capi.csr_spmm(crow.to(DEV), col.to(DEV), val.to(DEV), b.to(DEV), rows)
+    torch.cuda.synchronize()
+    _check(c, want, floor, "csr")
+    coo = a.to_sparse_coo().coalesce()
+    idx = coo.indices()
+    c2 = capi.coo_spmm(idx[0].contiguous().to(DEV), idx[1].contiguous().to(DEV), coo.values().to(DEV), b.to(DEV), rows)
+    torch.cuda.synchronize()
+    _check(c2, want, floor, "coo")
+
+
+def test_coo_unsorted_with_duplicates_and_strided_b():
+    from mamtorch_amd import capi
+
+    rows, k, cols = 70, 90, 48
+    g = torch.Generator().manual_seed(3)
+    nnz = 2000
+    row = torch.randint(0, rows, (nnz,), generator=g)
+    col = torch.randint(0, k, (nnz,), generator=g)
+    val = torch.randn(nnz, generator=g)
+    wide = torch.randn(k, cols + 16, generator=g)
+    b = wide[:, 8:8 + cols]                      # a view: row stride cols + 16, 32-byte offset
+    want, floor = oracle.coo_spmm(row.numpy(), col.numpy(), val.numpy(), b.contiguous().numpy(), rows)
+    bd = wide.to(DEV)[:, 8:8 + cols]
+    c = capi.coo_spmm(row.to(DEV), col.to(DEV), val.to(DEV), bd, rows)
+    torch.cuda.synchronize()
+    _check(c, want, floor, "coo unsorted")
+    # the same matrix through CSR with unsorted columns inside the rows
+    order = torch.argsort(row, stable=True)
+    crow = torch.zeros(rows + 1, dtype=torch.int64)
+    crow[1:] = torch.cumsum(torch.bincount(row, minlength=rows), 0)
+    c2 = capi.csr_spmm(crow.to(DEV), col[order].to(DEV), val[order].to(DEV), bd, rows)
+    torch.cuda.synchronize()
+    _check(c2, want, floor, "csr unsorted columns")
+
+
+@pytest.mark.parametrize("layout", [torch.sparse_csr, torch.sparse_coo])
+def test_operator_name_keys_and_reference_style_check(layout):
+    """The reference's own check (test/test_sparse.py:21-44) with seeds: random sizes in [10, 1000], 90 %
+    zeros, result against the dense product."""
+    import mamtorch_amd as mt
+
+    rng = np.random.default_rng(7)
+    n, l, m = (int(v) for v in rng.integers(10, 1000, 3))
+    a = _random_sparse(n, l, 0.9, seed=n).to(DEV)
+    b = torch.randn(l, m, generator=torch.Generator().manual_seed(m)).to(DEV)
+    asparse = a.to_sparse(layout=layout)
+    res = torch.ops.mamtorch_kernel_sparsev1.cusparsemm(asparse, b)
+    assert res.shape == (n, m) and res.dtype == torch.float32 and res.device == b.device
+    res2 = mt.sparse.kernel.v1.cusparsemm(asparse, b)
+    want = a.double() @ b.double()
+    floor = a.abs().double() @ b.abs().double()
+    for r in (res, res2):
+        assert bool(((r.double() - want).abs() <= 1e-5 * want.abs() + 2.0 ** -22 * floor).all())
+    with pytest.raises(RuntimeError):
+        torch.ops.mamtorch_kernel_sparsev1.cusparsemm(asparse, b[:-1])
+
+
+def test_full_size_against_dense_matmul():
+    from mamtorch_amd import capi
+
+    n = 4096
+    a = _random_sparse(n, n, 0.9, seed=1).to(DEV)
+    b = torch.randn(n, n, generator=torch.Generator().manual_seed(2)).to(DEV)
+    csr = a.to_sparse_csr()
+    c = capi.csr_spmm(csr.crow_indices(), csr.col_indices(), csr.values(), b, n)
+    want = a.double() @ b.double()
+    floor = a.abs().double() @ b.abs().double()
+    assert bool(((c.double() - want).abs() <= 1e-5 * want.abs() + 2.0 ** -22 * floor).all())
+    # linearity, a size-independent property: (2A) @ b == 2 (A @ b) bit for bit (scaling by 2 is exact)
+    c2 = capi.csr_spmm(csr.crow_indices(), csr.col_indices(), csr.values() * 2, b, n)
+    assert torch.equal(c2, c * 2)

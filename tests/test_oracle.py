@@ -242,3 +242,38 @@ def test_csr_oracle_equals_dense_on_densified_weight(density):
     np.testing.assert_allclose(xg, xd, rtol=1e-6, atol=1e-7)
     rows = np.repeat(np.arange(M), np.diff(crow.numpy()))
     np.testing.assert_allclose(vg, wd[rows, col.numpy()], rtol=1e-6, atol=1e-7)
+
+
+# ---- sum-of-products SpMM oracle (checker of mamtorch_kernel_sparsev1::cusparsemm) ----
+def _random_sparse(rows, k, sparse_rate, seed):
+    # the generator of the reference's own check, seeded (test/test_sparse.py:14-17)
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(rows, k, generator=g)
+    return a * torch.bernoulli(torch.full((rows, k), 1 - sparse_rate), generator=g)
+
+
+@pytest.mark.parametrize("rows,k,cols,rate", [(37, 53, 29, 0.9), (200, 310, 64, 0.7), (5, 1, 3, 0.0), (64, 64, 100, 0.99)])
+def test_spmm_oracle_against_dense_matmul_and_scipy(rows, k, cols, rate):
+    import scipy.sparse as sp
+
+    a = _random_sparse(rows, k, rate, seed=rows)
+    b = torch.randn(k, cols, generator=torch.Generator().manual_seed(k))
+    csr = a.to_sparse_csr()
+    got, floor = oracle.csr_spmm(csr.crow_indices().numpy(), csr.col_indices().numpy(), csr.values().numpy(), b.numpy())
+    want = a.numpy().astype(np.float64) @ b.numpy().astype(np.float64)
+    assert np.abs(got - want).max() <= 1e-6 * np.abs(want).max() + 1e-30
+    np.testing.assert_allclose(floor, np.abs(a.numpy()).astype(np.float64) @ np.abs(b.numpy()).astype(np.float64), rtol=1e-6)
+    lib_result = sp.csr_matrix((csr.values().numpy().astype(np.float64), csr.col_indices().numpy(),
+                                csr.crow_indices().numpy()), shape=(rows, k)) @ b.numpy().astype(np.float64)
+    assert np.abs(got - lib_result).max() <= 1e-6 * np.abs(want).max() + 1e-30
+
+
+def test_spmm_oracle_coo_any_order_and_duplicates():
+    # hand-derived: [[1,0,2],[0,0,0],[0,3,0]] with the (0,2) entry given as 0.5 + 1.5 and shuffled order
+    row = np.array([2, 0, 0, 0], dtype=np.int64)
+    col = np.array([1, 2, 0, 2], dtype=np.int64)
+    val = np.array([3.0, 0.5, 1.0, 1.5], dtype=np.float32)
+    b = np.array([[1.0, 2.0], [3.0, 4.0], [5.0, -6.0]], dtype=np.float32)
+    c, floor = oracle.coo_spmm(row, col, val, b, 3)
+    np.testing.assert_array_equal(c, np.array([[11.0, -10.0], [0.0, 0.0], [9.0, 12.0]], dtype=np.float32))
+    np.testing.assert_array_equal(floor, np.array([[11.0, 14.0], [0.0, 0.0], [9.0, 12.0]], dtype=np.float32))
