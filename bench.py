@@ -21,6 +21,8 @@ Other workloads (`--workload`), same JSON layout, used for the tables in the des
   sparse_d{10,03,01} 4096x4096 weight pruned to 10 % / 3 % / 1 %, batch 256, CSR forward + backward
   spmm_d{30,10,01}   sum-of-products SpMM (cusparsemm): 4096x4096 CSR with 30 % / 10 % / 1 % stored, times a
                      dense 4096x4096; one op = one multiply-add; torch.sparse.mm timed beside it
+  prune_csr          magnitude pruning of a 4096x4096 weight to 10 % and its compaction to CSR (row offsets +
+                     fill); one op = one weight examined; Tensor.to_sparse_csr of the masked weight timed beside it
 """
 import argparse
 import ctypes
@@ -42,7 +44,7 @@ FORWARD_TRAFFIC_BYTES = {"mam_fwd_kernel": 141.1e6, "mam_fwd_merge_kernel": 167.
 BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 103.4e6}
 
 WORKLOADS = ("headline", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
-             "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01")
+             "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01", "prune_csr")
 
 
 class Layer:
@@ -363,6 +365,54 @@ def run_spmm(torch, capi, lib, dev, args):
     return ops, ms_step, out, cpu
 
 
+def run_prune(torch, capi, lib, dev, args):
+    """prune_csr: |w| <= threshold goes (90 % of a N(0, 0.02) weight), survivors compacted to CSR."""
+    M = K = 4096
+    w = (torch.randn(M, K, generator=torch.Generator().manual_seed(0)) * 0.02).to(dev)
+    thr = float(torch.sort(w.flatten().abs())[0][int(0.9 * M * K)])
+    crow = torch.empty(M + 1, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    f = ctypes.c_float(thr)
+
+    def offsets():
+        rc = lib.mam_prune_row_offsets(P(w), K, capi.PRUNE_MAGNITUDE, None, None, K, f, P(crow), M, K, sp)
+        assert rc == 0, lib.mam_last_error()
+
+    offsets()
+    nnz = int(crow[M].item())
+    col = torch.empty(nnz, dtype=torch.int64, device=dev)
+    val = torch.empty(nnz, dtype=torch.float32, device=dev)
+
+    def fill():
+        rc = lib.mam_prune_fill_csr(P(w), K, capi.PRUNE_MAGNITUDE, None, None, K, f, P(crow), P(col), P(val), M, K, sp)
+        assert rc == 0, lib.mam_last_error()
+
+    ms_step, ph = time_phases(torch, stream, [("row_offsets", offsets), ("fill", fill)], args.steps, args.warmup)
+    masked = torch.where(w.abs() > thr, w, torch.zeros_like(w))
+    _, ph_lib = time_phases(torch, stream, [("Tensor.to_sparse_csr", lambda: masked.to_sparse_csr())],
+                            max(args.steps // 10, 5), 3)
+    nbytes = 2 * 4 * M * K + 8 * (M + 1) + 12 * nnz
+    out = {
+        "config": {"workload": "magnitude pruning of a 4096x4096 fp32 weight ~N(0,0.02) at the 90 % quantile and "
+                               "compaction of the survivors to CSR (int64 indices); one op = one weight examined",
+                   "name": args.workload, "M": M, "K": K, "nnz": nnz},
+        "phases_ms": {k: round(v, 5) for k, v in ph.items()},
+        "library_ms": {k: round(v, 5) for k, v in ph_lib.items()},
+        "roofline": hbm_roofline("prune count_kernel + scan_kernel + fill_kernel", nbytes, ms_step),
+    }
+    cpu = None
+    if args.cpu_seconds > 0:
+        wc = w.cpu()
+        t0 = time.perf_counter()
+        torch.where(wc.abs() > thr, wc, torch.zeros_like(wc)).to_sparse_csr()
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(M * K / dt / 1e9, 4), "unit": "GOPS", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": "mask + Tensor.to_sparse_csr of the whole weight on the CPU (%.2f s)" % dt}
+    return M * K, ms_step, out, cpu
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -376,7 +426,7 @@ def main():
         print("bench.py measures one GPU: the MAM hot path has no multi-GPU part in this build "
               "(--gpus %d refused)" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    small = args.workload in ("headline", "values_headline") or args.workload.startswith("sparse")
+    small = args.workload in ("headline", "values_headline", "prune_csr") or args.workload.startswith("sparse")
     if args.workload.startswith("spmm"):
         args.steps = 50 if args.steps is None else args.steps
         args.warmup = 20 if args.warmup is None else args.warmup
@@ -395,7 +445,7 @@ def main():
     dev = torch.device("cuda:0")
     lib = capi.lib()
     run = run_sparse if args.workload.startswith("sparse") else run_spmm if args.workload.startswith("spmm") \
-        else run_dense
+        else run_prune if args.workload == "prune_csr" else run_dense
     triples, ms_step, extra, cpu = run(torch, capi, lib, dev, args)
 
     out = {

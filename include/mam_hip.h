@@ -37,6 +37,10 @@ extern "C" {
 #define MAM_W_KM 0
 #define MAM_W_MK 1
 
+#define MAM_PRUNE_MAGNITUDE 0    /* score = |w|                                  */
+#define MAM_PRUNE_WEIGHT_TIMES 1 /* score = |w * aux|, aux (M,K) fp32 (e.g. w.grad) */
+#define MAM_PRUNE_COUNT 2        /* score = aux (+ aux2), (M,K) int32 selection counts */
+
 #define MAM_COUNT_REFERENCE 0 /* per call: +1 per (m,k) picked as max by >=1 row, +1 if picked as
                                  min by >=1 row, both into max_count (the module's literal rule) */
 #define MAM_COUNT_HITS 1      /* true hit counts: max_count += #argmax hits, min_count += #argmin */
@@ -143,6 +147,27 @@ int mam_csr_spmm(const int64_t *crow, const int64_t *col, const float *val, cons
                  float *c, int64_t R, int64_t K, int64_t C, void *stream);
 int mam_coo_spmm(const int64_t *row, const int64_t *col, const float *val, int64_t nnz, const float *b,
                  int64_t ldb, float *c, int64_t R, int64_t K, int64_t C, void *stream);
+
+/*
+ * Pruning of a dense weight w (M,K), row stride ldw, and its compaction to CSR.  An entry is pruned when
+ * its score is not above `threshold` -- the reference's `w[score.abs() <= threshold] = 0`
+ * (examples/vitb16_imagenet1k/pruning_utils.py:103-111 magnitude, :190-203 weight x gradient) -- and the
+ * score is chosen by `mode` (MAM_PRUNE_*); `aux` / `aux2` are (M,K) arrays of row stride ld_aux (aux2 only
+ * for MAM_PRUNE_COUNT, may be NULL): the counters kept by mam_selection_count
+ * (mamtorch/nn/v4/fullyconnected.py:107-131) are the third score.
+ *   mam_prune_row_offsets : crow (M+1) int64 = CSR row offsets of the survivors; nnz = crow[M]
+ *   mam_prune_fill_csr    : col (nnz) int64 ascending per row and val (nnz) fp32, for the same arguments
+ *   mam_prune_apply       : the reference's in-place form, pruned entries of w become 0.0f
+ * The reference itself keeps pruned weights dense; the CSR operands are what mam_csr_fc_forward and
+ * mam_csr_spmm take.
+ */
+int mam_prune_row_offsets(const float *w, int64_t ldw, int mode, const void *aux, const void *aux2,
+                          int64_t ld_aux, float threshold, int64_t *crow, int64_t M, int64_t K, void *stream);
+int mam_prune_fill_csr(const float *w, int64_t ldw, int mode, const void *aux, const void *aux2,
+                       int64_t ld_aux, float threshold, const int64_t *crow, int64_t *col, float *val,
+                       int64_t M, int64_t K, void *stream);
+int mam_prune_apply(float *w, int64_t ldw, int mode, const void *aux, const void *aux2, int64_t ld_aux,
+                    float threshold, int64_t M, int64_t K, void *stream);
 
 #ifdef __cplusplus
 }

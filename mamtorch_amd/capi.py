@@ -12,6 +12,9 @@ from . import _native
 
 W_KM = 0
 W_MK = 1
+PRUNE_MAGNITUDE = 0
+PRUNE_WEIGHT_TIMES = 1
+PRUNE_COUNT = 2
 COUNT_REFERENCE = 0
 COUNT_HITS = 1
 
@@ -22,6 +25,7 @@ EXPORTS = (
     "mam_fc_backward", "mam_selection_count",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward",
     "mam_csr_spmm", "mam_coo_spmm",
+    "mam_prune_row_offsets", "mam_prune_fill_csr", "mam_prune_apply",
 )
 
 _i64 = ctypes.c_int64
@@ -56,6 +60,10 @@ def lib():
                                           _ptr, _i64, _i64, _i64, _i64, _ptr]
         l.mam_csr_spmm.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
         l.mam_coo_spmm.argtypes = [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
+        _f = ctypes.c_float
+        l.mam_prune_row_offsets.argtypes = [_ptr, _i64, _int, _ptr, _ptr, _i64, _f, _ptr, _i64, _i64, _ptr]
+        l.mam_prune_fill_csr.argtypes = [_ptr, _i64, _int, _ptr, _ptr, _i64, _f, _ptr, _ptr, _ptr, _i64, _i64, _ptr]
+        l.mam_prune_apply.argtypes = [_ptr, _i64, _int, _ptr, _ptr, _i64, _f, _i64, _i64, _ptr]
         _configured = True
     return l
 
@@ -191,3 +199,43 @@ def coo_spmm(row, col, val, b, R):
     with torch.cuda.device(b.device):
         _check(l.mam_coo_spmm(_p(row), _p(col), _p(val), val.numel(), _p(b), _ld(b), _p(c), R, K, C, _stream(b)))
     return c
+
+
+def _prune_operands(w, mode, aux, aux2):
+    if mode == PRUNE_MAGNITUDE:
+        return None, None, max(w.size(1), 1)
+    want = torch.float32 if mode == PRUNE_WEIGHT_TIMES else torch.int32
+    for t in (aux, aux2):
+        if t is not None and (t.dtype != want or t.shape != w.shape or t.device != w.device or t.stride(1) != 1):
+            raise ValueError("score operand must be a %s tensor shaped and placed like the weight" % want)
+    if aux is None or (aux2 is not None and (mode != PRUNE_COUNT or _ld(aux2) != _ld(aux))):
+        raise ValueError("score operand missing or second operand not allowed")
+    return aux, aux2, _ld(aux)
+
+
+def prune_to_csr(w, threshold, mode=PRUNE_MAGNITUDE, aux=None, aux2=None):
+    """CSR parts (crow, col, val) of the entries of w (M, K) whose score is above `threshold`.
+    Reads crow[M] back to size col / val: the only host synchronisation."""
+    l = lib()
+    M, K = w.shape
+    aux, aux2, ld_aux = _prune_operands(w, mode, aux, aux2)
+    crow = torch.empty(M + 1, dtype=torch.int64, device=w.device)
+    with torch.cuda.device(w.device):
+        _check(l.mam_prune_row_offsets(_p(w), _ld(w), mode, _p(aux), _p(aux2), ld_aux, threshold, _p(crow), M, K,
+                                       _stream(w)))
+        nnz = int(crow[M].item())
+        col = torch.empty(nnz, dtype=torch.int64, device=w.device)
+        val = torch.empty(nnz, dtype=torch.float32, device=w.device)
+        _check(l.mam_prune_fill_csr(_p(w), _ld(w), mode, _p(aux), _p(aux2), ld_aux, threshold, _p(crow), _p(col),
+                                    _p(val), M, K, _stream(w)))
+    return crow, col, val
+
+
+def prune_apply(w, threshold, mode=PRUNE_MAGNITUDE, aux=None, aux2=None):
+    """In place: entries of w whose score is not above `threshold` become 0."""
+    l = lib()
+    M, K = w.shape
+    aux, aux2, ld_aux = _prune_operands(w, mode, aux, aux2)
+    with torch.cuda.device(w.device):
+        _check(l.mam_prune_apply(_p(w), _ld(w), mode, _p(aux), _p(aux2), ld_aux, threshold, M, K, _stream(w)))
+    return w

@@ -6,6 +6,7 @@ does not have, keep that operator's CSR operand convention (int64 crow/col, fp32
 operand dispatched on the sparse-CSR key).
 """
 from . import kernel
+from . import prune
 from .fullyconnected import fullyconnected, fullyconnected_backward, SparseFullyConnectedFunction, prune_to_csr
 
-__all__ = ["kernel", "fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr"]
+__all__ = ["kernel", "prune", "fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr"]

@@ -277,3 +277,41 @@ def test_spmm_oracle_coo_any_order_and_duplicates():
     c, floor = oracle.coo_spmm(row, col, val, b, 3)
     np.testing.assert_array_equal(c, np.array([[11.0, -10.0], [0.0, 0.0], [9.0, 12.0]], dtype=np.float32))
     np.testing.assert_array_equal(floor, np.array([[11.0, 14.0], [0.0, 0.0], [9.0, 12.0]], dtype=np.float32))
+
+
+# ---- pruning rule and dense -> CSR compaction oracle ----
+def test_prune_oracle_hand_derived():
+    from oracle import prune as po
+
+    w = np.array([[0.5, -0.2, 0.0, 0.3], [-0.3, 0.31, 0.29, -1.0]], dtype=np.float32)
+    crow, col, val = po.to_csr(w, 0.3)                     # |w| <= 0.3 goes: ties at the threshold go too
+    np.testing.assert_array_equal(crow, [0, 1, 3])
+    np.testing.assert_array_equal(col, [0, 1, 3])
+    np.testing.assert_array_equal(val, np.array([0.5, 0.31, -1.0], dtype=np.float32))
+    g = np.array([[1.0, 10.0, 5.0, -1.0], [0.0, 1.0, 2.0, 0.1]], dtype=np.float32)
+    np.testing.assert_array_equal(po.apply(w, 0.3, po.WEIGHT_TIMES, g),
+                                  np.array([[0.5, -0.2, 0.0, 0.0], [0.0, 0.31, 0.29, 0.0]], dtype=np.float32))
+    a = np.array([[0, 2, 1, 0], [3, 0, 0, 1]], dtype=np.int32)
+    b = np.array([[0, 0, 0, 1], [0, 0, 1, 0]], dtype=np.int32)
+    np.testing.assert_array_equal(po.keep_mask(w, 1.0, po.COUNT, a, b),
+                                  [[False, True, False, False], [True, False, False, False]])
+
+
+@pytest.mark.parametrize("p", [0.0, 0.5, 0.9, 0.99])
+def test_prune_oracle_against_the_literal_torch_rule(p):
+    from oracle import prune as po
+
+    g = torch.Generator().manual_seed(int(p * 100))
+    w = torch.randn(37, 101, generator=g) * 0.02
+    grad = torch.randn(37, 101, generator=g)
+    for mode, score in ((po.MAGNITUDE, w), (po.WEIGHT_TIMES, w * grad)):
+        thr = float(torch.quantile(score.flatten().abs(), p))      # pruning_utils.py:104
+        want = w.clone()
+        want[score.abs() <= thr] = 0                                # pruning_utils.py:105
+        np.testing.assert_array_equal(po.apply(w.numpy(), thr, mode, grad.numpy()), want.numpy())
+        crow, col, val = po.to_csr(w.numpy(), thr, mode, grad.numpy())
+        csr = want.to_sparse_csr()                                  # drops the zeros the rule wrote
+        kept_nonzero = val != 0
+        np.testing.assert_array_equal(col[kept_nonzero], csr.col_indices().numpy())
+        np.testing.assert_array_equal(val[kept_nonzero], csr.values().numpy())
+        assert crow[-1] == len(col) and abs(len(col) / w.numel() - (1 - p)) < 0.02
