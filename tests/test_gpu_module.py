@@ -215,3 +215,40 @@ def test_sparse_operator_and_autograd_function():
                                  w2.values().cpu().numpy(), grad.numpy(), want[1], want[2])
     np.testing.assert_allclose(xin.grad.cpu().numpy(), xo, rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(vals.grad.cpu().numpy(), vo, rtol=1e-5, atol=1e-6)
+
+
+def test_linear_layers_swapped_for_mam_and_vit_mlp_block():
+    """examples/vitb16_imagenet1k/utils.py:67-77: the swapped layer starts from the Linear's weight and
+    bias; the ViT-B/16 MLP block (768 -> 3072 -> 768) on 2 x 197 tokens against the oracle, layer by layer."""
+    torch.manual_seed(0)
+    model = torch.nn.Sequential()
+    model.add_module("encoder", torch.nn.Module())
+    model.encoder.intermediate = torch.nn.Linear(64, 96)
+    model.encoder.output = torch.nn.Linear(96, 64, bias=False)
+    model.encoder.keep = torch.nn.Linear(8, 8)
+    w1, b1 = model.encoder.intermediate.weight.data.clone(), model.encoder.intermediate.bias.data.clone()
+    mt.nn.add_mam_to_model(model, ["encoder.intermediate", "encoder.output"], vcon_steps=4, store_args=True)
+    assert isinstance(model.encoder.intermediate, mt.nn.FullyConnected)
+    assert isinstance(model.encoder.output, mt.nn.FullyConnected) and model.encoder.output.bias is None
+    assert isinstance(model.encoder.keep, torch.nn.Linear)
+    assert torch.equal(model.encoder.intermediate.weight.data, w1) and torch.equal(model.encoder.intermediate.bias.data, b1)
+    assert model.encoder.intermediate.beta == 1.0 and model.encoder.intermediate.vcon_steps == 4
+    assert mt.nn.get_layers(model, ["encoder.keep"])[0] is model.encoder.keep
+    with pytest.raises(TypeError):
+        mt.nn.add_mam_to_model(model, ["encoder.output"])
+
+    block = mt.nn.MAMMlp().to(DEV)
+    tokens = torch.randn(2, 197, 768, generator=torch.Generator().manual_seed(1)).to(DEV).requires_grad_(True)
+    out = block(tokens)
+    assert out.shape == tokens.shape
+    normed = block.norm(tokens.detach()).detach().reshape(-1, 768)
+    c1 = oracle.forward(normed.cpu().numpy(), block.intermediate.weight.detach().cpu().numpy(), oracle.W_MK,
+                        block.intermediate.bias.detach().cpu().numpy())[0]
+    h = F.gelu(torch.from_numpy(c1).to(DEV))
+    c2 = oracle.forward(h.cpu().numpy(), block.output.weight.detach().cpu().numpy(), oracle.W_MK,
+                        block.output.bias.detach().cpu().numpy())[0]
+    want = tokens.detach().reshape(-1, 768) + torch.from_numpy(c2).to(DEV)
+    assert_bits_equal(out.detach().reshape(-1, 768).cpu().numpy(), want.cpu().numpy(), "MLP block output")
+    out.sum().backward()
+    assert tokens.grad is not None and block.intermediate.weight.grad is not None
+    assert torch.isfinite(tokens.grad).all()
