@@ -35,6 +35,9 @@
 // ascending k order with the same strict comparisons before resolving indices.
 #include "mam_common.h"
 
+#include <stdlib.h>
+#include <string.h>
+
 namespace mam {
 namespace fwd {
 
@@ -663,10 +666,221 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
     }
 }
 
-// How many K ranges to split into so that at least two workgroups reach every CU.
-static int choose_splits(int64_t N, int64_t K, int64_t M)
+
+// ---------------------------------------------------------------------------------------------
+// Second tiling for the (M,K) layout with whole 32-k tiles: batch rows are wave-uniform.
+//
+// A wave owns 4 batch rows x 256 neurons (lane + 64 j): its x operands are the same for all
+// lanes, so they come through the scalar cache into SGPRs (a VALU multiply takes one SGPR
+// operand at no cost) and occupy no vector register and no LDS read.  What a thread holds is
+// 16 outputs x (max, min, two group ids) + one W column of 16 k: under 128 VGPRs, four waves
+// per SIMD, so a wave that waits (LDS, barrier, scalar load) leaves three to issue from.  Eight
+// waves = 32 batch rows share one W tile of 256 neurons x 32 k (32 KiB, two of them in flight,
+// two workgroups per CU).  The tile is stored [neuron][k] without padding; 16-byte chunk c of
+// neuron r sits at chunk c ^ ((r >> 1) & 7), which spreads a ds_read_b128 of 16 consecutive
+// neurons over all banks, and since direct-to-LDS loads write LDS linearly the permutation is
+// applied to the global addresses instead.
+namespace sx {
+constexpr int BN = 32;    // batch rows per workgroup
+constexpr int BM = 256;   // neurons per workgroup
+constexpr int NT = 512;   // threads per workgroup
+constexpr int TI = 4;     // batch rows per wave
+constexpr int TJ = 4;     // neurons per lane
+constexpr int TILE_FLOATS = BM * KT;
+constexpr int DMA_INSTR = TILE_FLOATS / 256;          // wave-level 1 KiB loads per tile
+constexpr int DMA_PER_WAVE = DMA_INSTR / (NT / 64);
+static_assert(DMA_PER_WAVE * (NT / 64) == DMA_INSTR, "tile must split evenly over the waves");
+}  // namespace sx
+
+typedef const __attribute__((address_space(4))) float const_f32;
+
+template <bool ARGS, bool SPLIT>
+__global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 {
-    const int64_t tiles = ceil_div(N, BN) * ceil_div(M, BM);
+    __shared__ __attribute__((aligned(16))) float tile_a[sx::TILE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float tile_b[sx::TILE_FLOATS];
+    __shared__ uint32_t doff_s[sx::DMA_PER_WAVE * sx::NT];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // ---- which tile: as in the first tiling ----
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int tiles = p.tiles_n * p.tiles_m;
+    const int split = logical / tiles;
+    const int l = logical - split * tiles;
+    const int per_group = GROUP_N * p.tiles_m;
+    const int grp = l / per_group;
+    const int first_n = grp * GROUP_N;
+    const int gsize = (p.tiles_n - first_n) < GROUP_N ? (p.tiles_n - first_n) : GROUP_N;
+    const int lin = l - grp * per_group;
+    const int tn = first_n + lin % gsize;
+    const int tm = lin / gsize;
+    const int row0 = tn * sx::BN + sx::TI * wave, col0 = tm * sx::BM;
+    const int kb = split * p.k_per_split;
+    const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
+    const int ntiles = (ke - kb) / KT;    // the host sends only whole tiles here
+
+    float vmax[sx::TI][sx::TJ], vmin[sx::TI][sx::TJ];
+    int gmax[sx::TI][sx::TJ], gmin[sx::TI][sx::TJ];
+#pragma unroll
+    for (int i = 0; i < sx::TI; ++i)
+#pragma unroll
+        for (int j = 0; j < sx::TJ; ++j) {
+            vmax[i][j] = -__builtin_inff();
+            vmin[i][j] = __builtin_inff();
+            gmax[i][j] = 0;
+            gmin[i][j] = 0;
+        }
+
+    // rows past the batch repeat the last one (never stored)
+    const_f32 *xr[sx::TI];
+#pragma unroll
+    for (int i = 0; i < sx::TI; ++i) {
+        const int row = (row0 + i) < p.N ? (row0 + i) : (p.N - 1);
+        xr[i] = (const_f32 *)(p.x + (int64_t)row * p.ldx + kb);
+    }
+
+    // per-lane byte offsets of this wave's direct-to-LDS loads, kept in LDS
+    const uint32_t *doff = doff_s + tid;
+#pragma unroll
+    for (int t = 0; t < sx::DMA_PER_WAVE; ++t) {
+        const int inst = wave + (sx::NT / 64) * t;
+        const int r = inst * 8 + (lane >> 3);               // neuron within the tile
+        const int chunk = (lane & 7) ^ ((r >> 1) & 7);      // the k chunk that belongs at this LDS position
+        const int rc = ((col0 + r) < p.M ? (col0 + r) : (p.M - 1)) - col0;
+        doff_s[t * sx::NT + tid] = (uint32_t)(rc * (int)p.ldw + chunk * 4) * 4u;
+    }
+    const int sw = (lane >> 1) & 7;
+    const int wbase = lane * KT;     // floats; neuron lane + 64 j is 64 j * KT further
+
+    auto dma = [&](const char *wk, float *tile) {
+#pragma unroll
+        for (int t = 0; t < sx::DMA_PER_WAVE; ++t) {
+            const int inst = wave + (sx::NT / 64) * t;
+            const char *src = wk + (uint64_t)doff[t * sx::NT];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)(tile + inst * 256), 16, 0, 0);
+        }
+    };
+    auto compute = [&](const float *tile, int t) {
+#pragma unroll
+        for (int gg = 0; gg < KT / G; ++gg) {
+            const int grel = t * (KT / G) + gg;
+            float xv[sx::TI][G];
+#pragma unroll
+            for (int i = 0; i < sx::TI; ++i)
+#pragma unroll
+                for (int q = 0; q < G; ++q) xv[i][q] = xr[i][t * KT + gg * G + q];
+#pragma unroll
+            for (int j = 0; j < sx::TJ; ++j) {
+                float wv[G];
+#pragma unroll
+                for (int q = 0; q < G / 4; ++q) {
+                    const float4 v = *reinterpret_cast<const float4 *>(
+                        &tile[wbase + 64 * j * KT + (((gg * (G / 4) + q) ^ sw) << 2)]);
+                    wv[q * 4 + 0] = v.x; wv[q * 4 + 1] = v.y; wv[q * 4 + 2] = v.z; wv[q * 4 + 3] = v.w;
+                }
+#pragma unroll
+                for (int i = 0; i < sx::TI; ++i) {
+                    const float om = vmax[i][j], on = vmin[i][j];
+                    float hi = om, lo = on;
+#pragma unroll
+                    for (int q = 0; q < G; q += 2) {
+                        const float a = xv[i][q] * wv[q], b = xv[i][q + 1] * wv[q + 1];
+                        hi = __builtin_fmaxf(__builtin_fmaxf(hi, a), b);
+                        lo = __builtin_fminf(__builtin_fminf(lo, a), b);
+                    }
+                    if (ARGS) {
+                        gmax[i][j] = (hi > om) ? grel : gmax[i][j];
+                        gmin[i][j] = (lo < on) ? grel : gmin[i][j];
+                    }
+                    vmax[i][j] = hi;
+                    vmin[i][j] = lo;
+                }
+            }
+        }
+    };
+
+    const char *wk = reinterpret_cast<const char *>(p.w + (int64_t)col0 * p.ldw + kb);
+    if (ntiles > 0) {
+        dma(wk, tile_a);
+        __syncthreads();
+        for (int t = 0; t < ntiles; t += 2) {
+            wk += KT * sizeof(float);
+            if (t + 1 < ntiles) dma(wk, tile_b);
+            compute(tile_a, t);
+            __syncthreads();
+            if (t + 1 >= ntiles) break;
+            wk += KT * sizeof(float);
+            if (t + 2 < ntiles) dma(wk, tile_a);
+            compute(tile_b, t + 1);
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue ----
+    const int g0 = kb / G;
+    if (SPLIT) {
+        const int64_t nm = (int64_t)p.N * p.M;
+        float *base = p.part + (int64_t)split * (ARGS ? 3 : 2) * nm;
+#pragma unroll
+        for (int i = 0; i < sx::TI; ++i)
+#pragma unroll
+            for (int j = 0; j < sx::TJ; ++j) {
+                const int n = row0 + i, m = col0 + lane + 64 * j;
+                if (n < p.N && m < p.M) {
+                    const int64_t o = (int64_t)n * p.M + m;
+                    base[o] = vmax[i][j];
+                    base[nm + o] = vmin[i][j];
+                    if (ARGS) base[2 * nm + o] = __int_as_float(gmax[i][j] | (gmin[i][j] << 16));
+                }
+            }
+    } else if (ARGS) {
+        // A wave parks one batch row (4 sets of 64 neurons) in its own corner of the dead tiles
+        // and resolves it set by set; the 64 outputs of a set share their x row.
+        float *vals = tile_a + wave * (sx::TJ * 128);
+        int *grps = reinterpret_cast<int *>(tile_b) + wave * (sx::TJ * 128);
+#pragma unroll
+        for (int i = 0; i < sx::TI; ++i) {
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < sx::TJ; ++j) {
+                vals[(j * 2 + 0) * 64 + lane] = vmax[i][j];
+                vals[(j * 2 + 1) * 64 + lane] = vmin[i][j];
+                grps[(j * 2 + 0) * 64 + lane] = g0 + gmax[i][j];
+                grps[(j * 2 + 1) * 64 + lane] = g0 + gmin[i][j];
+            }
+            __syncthreads();
+            const int nrow = row0 + i;
+#pragma unroll 1
+            for (int j = 0; j < sx::TJ; ++j) {
+                const int mbase = col0 + 64 * j;
+                resolve_wave(p, vals + j * 128, grps + j * 128, lane,
+                             [&](int slot, int &n, int &m, bool &valid) {
+                                 n = nrow;
+                                 m = mbase + slot;
+                                 valid = n < p.N && m < p.M;
+                                 n = n < p.N ? n : p.N - 1;
+                                 m = m < p.M ? m : p.M - 1;
+                             });
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < sx::TI; ++i)
+#pragma unroll
+            for (int j = 0; j < sx::TJ; ++j) {
+                const int n = row0 + i, m = col0 + lane + 64 * j;
+                if (n < p.N && m < p.M) finish<MAM_W_MK, false>(p, n, m, vmax[i][j], vmin[i][j], 0, 0);
+            }
+    }
+}
+
+// How many K ranges to split into so that at least two workgroups reach every CU.
+static int choose_splits(int64_t N, int64_t K, int64_t M, int bn = BN, int bm = BM)
+{
+    const int64_t tiles = ceil_div(N, bn) * ceil_div(M, bm);
     const int64_t want = 2 * kNumCU;
     if (tiles >= want) return 1;
     int64_t s = ceil_div(want, tiles);
@@ -681,7 +895,9 @@ static int choose_splits(int64_t N, int64_t K, int64_t M)
 
 static size_t workspace_bytes(int64_t N, int64_t K, int64_t M, bool args)
 {
-    const int s = choose_splits(N, K, M);
+    // whichever tiling the launch picks (it depends on alignment, unknown here): the larger need
+    const int s1 = choose_splits(N, K, M), s2 = choose_splits(N, K, M, sx::BN, sx::BM);
+    const int s = s1 > s2 ? s1 : s2;
     if (s == 1) return 0;
     return (size_t)s * (args ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float);
 }
@@ -707,9 +923,18 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     p.x = x; p.ldx = ldx; p.w = w; p.ldw = ldw; p.bias = bias;
     p.c = c; p.argmax = argmax; p.argmin = argmin; p.wsel = w_sel;
     p.N = (int)N; p.K = (int)K; p.M = (int)M;
-    p.tiles_n = (int)ceil_div(N, BN);
-    p.tiles_m = (int)ceil_div(M, BM);
-    p.splits = choose_splits(N, K, M);
+    p.vec_x = (ldx % 4 == 0) && ((uintptr_t)x % 16 == 0);
+    p.vec_w = (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0);
+    // The wave-uniform-rows tiling takes (M,K) weights with aligned rows and whole 32-k tiles; the
+    // environment variable MAM_FORWARD_TILING=wide keeps every shape on the first tiling (for
+    // comparisons and tests).
+    const char *tiling = getenv("MAM_FORWARD_TILING");
+    const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % KT == 0) &&
+                        (ldw * sx::BM < (1ll << 30)) && !(tiling && strcmp(tiling, "wide") == 0);
+    const int bn = use_sx ? sx::BN : BN, bm = use_sx ? sx::BM : BM;
+    p.tiles_n = (int)ceil_div(N, bn);
+    p.tiles_m = (int)ceil_div(M, bm);
+    p.splits = choose_splits(N, K, M, bn, bm);
     p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), KT) * KT);
     p.splits = (int)ceil_div(K, p.k_per_split);
     p.part = nullptr;
@@ -720,8 +945,6 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
                         workspace ? workspace_size : (size_t)0);
         p.part = static_cast<float *>(workspace);
     }
-    p.vec_x = (ldx % 4 == 0) && ((uintptr_t)x % 16 == 0);
-    p.vec_w = (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0);
     // the fast staging path addresses a tile with 32-bit element offsets from the tile base
     const int64_t w_rows = (w_layout == MAM_W_MK) ? fwd::BM : fwd::KT;
     p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30));
@@ -733,7 +956,11 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     const int64_t nblk = (int64_t)p.tiles_n * p.tiles_m * p.splits;
     if (nblk > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "too many tiles");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (w_layout == MAM_W_MK)
+    if (use_sx && p.splits > 1)
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<ARGS, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+    else if (use_sx)
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<ARGS, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+    else if (w_layout == MAM_W_MK)
         hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_MK, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
     else
         hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_KM, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);

@@ -26,12 +26,20 @@ def _run_both_layouts(x, w_mk, bias=None, what=""):
     want = oracle.forward(x.numpy(), w_mk.numpy(), oracle.W_MK, None if bias is None else bias.numpy())
     xd = x.to(dev)
     bd = None if bias is None else bias.to(dev)
-    for layout, w in ((capi.W_MK, w_mk.contiguous()), (capi.W_KM, w_mk.T.contiguous())):
+    # the (M,K) layout twice: the library picks its wave-uniform-rows tiling where the shape allows it;
+    # MAM_FORWARD_TILING=wide (read at every call) keeps it on the first tiling
+    for layout, w, tiling in ((capi.W_MK, w_mk.contiguous(), None), (capi.W_MK, w_mk.contiguous(), "wide"),
+                              (capi.W_KM, w_mk.T.contiguous(), None)):
         wd = w.to(dev)
-        c, amax, amin = capi.fc_forward(xd, wd, layout, bd)
-        cv = capi.fc_forward_values(xd, wd, layout, bd)
-        torch.cuda.synchronize()
-        tag = "%s layout=%d" % (what, layout)
+        if tiling:
+            os.environ["MAM_FORWARD_TILING"] = tiling
+        try:
+            c, amax, amin = capi.fc_forward(xd, wd, layout, bd)
+            cv = capi.fc_forward_values(xd, wd, layout, bd)
+            torch.cuda.synchronize()
+        finally:
+            os.environ.pop("MAM_FORWARD_TILING", None)
+        tag = "%s layout=%d tiling=%s" % (what, layout, tiling or "default")
         assert_bits_equal(c.cpu().numpy(), want[0], tag + " c")
         assert_index_equal(amax.cpu().numpy(), want[1], tag + " argmax")
         assert_index_equal(amin.cpu().numpy(), want[2], tag + " argmin")
