@@ -867,13 +867,38 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
             }
         }
     } else {
+        // values only: every thread parks its 16 results in its own LDS slots so that finishing them
+        // is one rolled loop (one copy of the code, no register array indexed at run time)
+        static_assert(sx::TI * sx::TJ * sx::NT <= sx::TILE_FLOATS, "result stash does not fit a tile buffer");
+        float *smax = tile_a + tid, *smin = tile_b + tid;
 #pragma unroll
         for (int i = 0; i < sx::TI; ++i)
 #pragma unroll
             for (int j = 0; j < sx::TJ; ++j) {
-                const int n = row0 + i, m = col0 + lane + 64 * j;
-                if (n < p.N && m < p.M) finish<MAM_W_MK, false>(p, n, m, vmax[i][j], vmin[i][j], 0, 0);
+                smax[(i * sx::TJ + j) * sx::NT] = vmax[i][j];
+                smin[(i * sx::TJ + j) * sx::NT] = vmin[i][j];
             }
+#pragma unroll 1
+        for (int o = 0; o < sx::TI * sx::TJ; ++o) {
+            const int n = row0 + o / sx::TJ, m = col0 + lane + 64 * (o % sx::TJ);
+            if (n < p.N && m < p.M) {
+                float hi = smax[o * sx::NT], lo = smin[o * sx::NT];
+                if (hi == 0.0f || lo == 0.0f) {
+                    // a zero extreme carries the sign of the first zero product (rare: plain scan)
+                    const float *xrow = p.x + (int64_t)n * p.ldx, *wrow = p.w + (int64_t)m * p.ldw;
+                    float z = 0.0f;
+                    for (int k = 0; k < p.K; ++k) {
+                        const float prod = xrow[k] * wrow[k];
+                        if (prod == 0.0f) { z = prod; break; }
+                    }
+                    hi = hi == 0.0f ? z : hi;
+                    lo = lo == 0.0f ? z : lo;
+                }
+                float sum = hi + lo;
+                if (p.bias) sum = sum + p.bias[m];
+                p.c[(int64_t)n * p.M + m] = sum;
+            }
+        }
     }
 }
 
