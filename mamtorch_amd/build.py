@@ -41,7 +41,9 @@ def build_hip(verbose=False):
 
     def compile_one(src):
         obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
-        out = _run([hipcc] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        # MAM_HIPFLAGS: extra compiler flags, e.g. -D switches of tuning constants
+        out = _run([hipcc] + HIP_FLAGS + os.environ.get("MAM_HIPFLAGS", "").split()
+                   + ["-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)
         return obj

@@ -668,24 +668,38 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
 
 
 // ---------------------------------------------------------------------------------------------
-// Second tiling for the (M,K) layout with whole 32-k tiles: batch rows are wave-uniform.
+// Second tiling for the (M,K) layout with whole 64-k tiles: batch rows are wave-uniform.
 //
-// A wave owns 4 batch rows x 256 neurons (lane + 64 j): its x operands are the same for all
+// A wave owns 4 batch rows x 128 neurons (lane + 64 j): its x operands are the same for all
 // lanes, so they come through the scalar cache into SGPRs (a VALU multiply takes one SGPR
-// operand at no cost) and occupy no vector register and no LDS read.  What a thread holds is
-// 16 outputs x (max, min, two group ids) + one W column of 16 k: under 128 VGPRs, four waves
-// per SIMD, so a wave that waits (LDS, barrier, scalar load) leaves three to issue from.  Eight
-// waves = 32 batch rows share one W tile of 256 neurons x 32 k (32 KiB, two of them in flight,
-// two workgroups per CU).  The tile is stored [neuron][k] without padding; 16-byte chunk c of
-// neuron r sits at chunk c ^ ((r >> 1) & 7), which spreads a ds_read_b128 of 16 consecutive
-// neurons over all banks, and since direct-to-LDS loads write LDS linearly the permutation is
-// applied to the global addresses instead.
+// operand at no cost) and occupy no vector register and no LDS read.  LDS reads per product
+// depend only on the rows per wave (one W value serves 4 products), not on the neurons per lane,
+// so a thread holds just 8 outputs x (max, min, two group ids) + one W column of 16 k: ~100
+// VGPRs, four waves per SIMD, and a wave that waits (LDS, barrier, scalar load) leaves three to
+// issue from.  Eight waves = 32 batch rows share one W tile of 128 neurons x 64 k (32 KiB, two of
+// them in flight, two workgroups per CU), one barrier per 64 k.  The tile is stored [neuron][k]
+// without padding; 16-byte chunk c of neuron r sits at chunk c ^ (r & 15), which spreads a
+// ds_read_b128 of 16 consecutive neurons over all banks, and since direct-to-LDS loads write LDS
+// linearly the permutation is applied to the global addresses instead.
+// Measured against the first tiling: 194 us against 216 us at the headline shape, 3.9 ms against
+// 4.9 ms for the two ViT MLP layers.  Neurons per lane / tile depth of 4 / 32 gave the same
+// headline time and 6 % more on the other shapes; reading the next W column ahead of its use
+// changed nothing.
 namespace sx {
+#ifndef MAM_SX_TJ
+#define MAM_SX_TJ 2
+#endif
+#ifndef MAM_SX_KT
+#define MAM_SX_KT 64
+#endif
 constexpr int BN = 32;    // batch rows per workgroup
-constexpr int BM = 256;   // neurons per workgroup
 constexpr int NT = 512;   // threads per workgroup
 constexpr int TI = 4;     // batch rows per wave
-constexpr int TJ = 4;     // neurons per lane
+constexpr int TJ = MAM_SX_TJ;     // neurons per lane
+constexpr int BM = 64 * TJ;       // neurons per workgroup
+constexpr int KT = MAM_SX_KT;     // k extent of one W tile
+constexpr int CHUNKS = KT / 4;    // 16-byte chunks per neuron and tile
+constexpr int RPB = 64 / KT < 1 ? 1 : 64 / KT;   // neurons per 256 bytes of LDS (all 64 banks)
 constexpr int TILE_FLOATS = BM * KT;
 constexpr int DMA_INSTR = TILE_FLOATS / 256;          // wave-level 1 KiB loads per tile
 constexpr int DMA_PER_WAVE = DMA_INSTR / (NT / 64);
@@ -719,7 +733,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     const int row0 = tn * sx::BN + sx::TI * wave, col0 = tm * sx::BM;
     const int kb = split * p.k_per_split;
     const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
-    const int ntiles = (ke - kb) / KT;    // the host sends only whole tiles here
+    const int ntiles = (ke - kb) / sx::KT;    // the host sends only whole tiles here
 
     float vmax[sx::TI][sx::TJ], vmin[sx::TI][sx::TJ];
     int gmax[sx::TI][sx::TJ], gmin[sx::TI][sx::TJ];
@@ -746,13 +760,14 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 #pragma unroll
     for (int t = 0; t < sx::DMA_PER_WAVE; ++t) {
         const int inst = wave + (sx::NT / 64) * t;
-        const int r = inst * 8 + (lane >> 3);               // neuron within the tile
-        const int chunk = (lane & 7) ^ ((r >> 1) & 7);      // the k chunk that belongs at this LDS position
+        const int r = inst * (64 / sx::CHUNKS) + lane / sx::CHUNKS;   // neuron within the tile
+        // the k chunk that belongs at this LDS position
+        const int chunk = (lane % sx::CHUNKS) ^ ((r / sx::RPB) & (sx::CHUNKS - 1));
         const int rc = ((col0 + r) < p.M ? (col0 + r) : (p.M - 1)) - col0;
         doff_s[t * sx::NT + tid] = (uint32_t)(rc * (int)p.ldw + chunk * 4) * 4u;
     }
-    const int sw = (lane >> 1) & 7;
-    const int wbase = lane * KT;     // floats; neuron lane + 64 j is 64 j * KT further
+    const int sw = (lane / sx::RPB) & (sx::CHUNKS - 1);   // the same for neurons lane + 64 j
+    const int wbase = lane * sx::KT;     // floats; neuron lane + 64 j is 64 j * KT further
 
     auto dma = [&](const char *wk, float *tile) {
 #pragma unroll
@@ -765,20 +780,20 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     };
     auto compute = [&](const float *tile, int t) {
 #pragma unroll
-        for (int gg = 0; gg < KT / G; ++gg) {
-            const int grel = t * (KT / G) + gg;
+        for (int gg = 0; gg < sx::KT / G; ++gg) {
+            const int grel = t * (sx::KT / G) + gg;
             float xv[sx::TI][G];
 #pragma unroll
             for (int i = 0; i < sx::TI; ++i)
 #pragma unroll
-                for (int q = 0; q < G; ++q) xv[i][q] = xr[i][t * KT + gg * G + q];
+                for (int q = 0; q < G; ++q) xv[i][q] = xr[i][t * sx::KT + gg * G + q];
 #pragma unroll
             for (int j = 0; j < sx::TJ; ++j) {
                 float wv[G];
 #pragma unroll
                 for (int q = 0; q < G / 4; ++q) {
                     const float4 v = *reinterpret_cast<const float4 *>(
-                        &tile[wbase + 64 * j * KT + (((gg * (G / 4) + q) ^ sw) << 2)]);
+                        &tile[wbase + 64 * j * sx::KT + (((gg * (G / 4) + q) ^ sw) << 2)]);
                     wv[q * 4 + 0] = v.x; wv[q * 4 + 1] = v.y; wv[q * 4 + 2] = v.z; wv[q * 4 + 3] = v.w;
                 }
 #pragma unroll
@@ -807,12 +822,12 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
         dma(wk, tile_a);
         __syncthreads();
         for (int t = 0; t < ntiles; t += 2) {
-            wk += KT * sizeof(float);
+            wk += sx::KT * sizeof(float);
             if (t + 1 < ntiles) dma(wk, tile_b);
             compute(tile_a, t);
             __syncthreads();
             if (t + 1 >= ntiles) break;
-            wk += KT * sizeof(float);
+            wk += sx::KT * sizeof(float);
             if (t + 2 < ntiles) dma(wk, tile_a);
             compute(tile_b, t + 1);
             __syncthreads();
@@ -954,13 +969,14 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     // environment variable MAM_FORWARD_TILING=wide keeps every shape on the first tiling (for
     // comparisons and tests).
     const char *tiling = getenv("MAM_FORWARD_TILING");
-    const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % KT == 0) &&
+    const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % sx::KT == 0) &&
                         (ldw * sx::BM < (1ll << 30)) && !(tiling && strcmp(tiling, "wide") == 0);
     const int bn = use_sx ? sx::BN : BN, bm = use_sx ? sx::BM : BM;
     p.tiles_n = (int)ceil_div(N, bn);
     p.tiles_m = (int)ceil_div(M, bm);
     p.splits = choose_splits(N, K, M, bn, bm);
-    p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), KT) * KT);
+    const int kt = use_sx ? sx::KT : KT;
+    p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), kt) * kt);
     p.splits = (int)ceil_div(K, p.k_per_split);
     p.part = nullptr;
     if (p.splits > 1) {
