@@ -24,7 +24,7 @@ def assert_index_equal(got, want, what):
 
 
 def config1(seed=0):
-    """BASELINE config 1: N64 K784 M256, bias on, Kaiming-uniform weight, seeded on the CPU."""
+    """The small CPU-runnable configuration: N64 K784 M256, bias on, Kaiming-uniform weight, seeded on the CPU."""
     g = torch.Generator().manual_seed(seed)
     N, K, M = 64, 784, 256
     bound = 1.0 / K ** 0.5

@@ -170,3 +170,16 @@ def test_selection_count_requires_store_args():
     layer.reset_selection_count()
     assert layer.max_selection_count.dtype == torch.int32 and layer.max_selection_count.shape == (4, 8)
     assert int(layer.min_selection_count.sum()) == 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU: any other --gpus value exits with a message before touching torch."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--workload", "nonsense"], capture_output=True,
+                       text=True)
+    assert r.returncode != 0
