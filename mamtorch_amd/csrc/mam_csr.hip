@@ -16,8 +16,8 @@
 // kernel, so exact tracking is affordable and nothing is re-scanned afterwards.
 // The lowest column missing from the row is found once per row; the
 // implicit-zero candidate x[n, missing] * 0 is compared last under the dense rule (greater wins,
-// equal -> lower index wins).  The four waves of a workgroup own four consecutive neurons and
-// hand their results over through LDS so that every batch row stores 16 contiguous bytes.
+// equal -> lower index wins).  The 16 waves of a workgroup own 16 consecutive neurons and hand
+// their results over through LDS so that every batch row stores 64 contiguous bytes per array.
 //
 // Backward: when the forward handed over the selected values and their entry positions, x_grad is the
 // dense x_grad kernel fed with those values (an implicit zero contributes 0), and val_grad is
@@ -34,7 +34,8 @@ namespace csr {
 constexpr int NT = 256;
 constexpr int NT_B = 512;  // backward workgroup
 constexpr int EG = 8;      // entries whose loads are issued together
-constexpr int ROWS = NT / 64;  // CSR rows per forward workgroup (one per wave)
+constexpr int NT_F = 1024;      // forward workgroup
+constexpr int ROWS = NT_F / 64;  // CSR rows per forward workgroup (one per wave)
 
 typedef const __attribute__((address_space(4))) int64_t const_i64;
 typedef const __attribute__((address_space(4))) float const_f32;
@@ -69,7 +70,7 @@ __device__ __forceinline__ float lane_elem(const float4 &v, int t)
 }
 
 template <int TI>
-__global__ __launch_bounds__(NT) void csr_fwd_kernel(
+__global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
     const float *__restrict__ xT, int ldt, const int64_t *__restrict__ crow,
     const int64_t *__restrict__ col, const float *__restrict__ val, const float *__restrict__ bias,
     float *__restrict__ c, int32_t *__restrict__ argmax, int32_t *__restrict__ argmin,
@@ -77,10 +78,15 @@ __global__ __launch_bounds__(NT) void csr_fwd_kernel(
 {
     typedef typename XVec<TI>::type xvec;
     constexpr int TILE_N = 64 * TI;
-    __shared__ float out_c[ROWS][TILE_N];
-    __shared__ int out_hi[ROWS][TILE_N], out_lo[ROWS][TILE_N];
-    __shared__ float out_wh[ROWS][TILE_N], out_wl[ROWS][TILE_N];
-    __shared__ int out_ph[ROWS][TILE_N], out_pl[ROWS][TILE_N];
+    // results of the workgroup's 16 neurons, [array][neuron][batch row]: 7 x 16 KiB for TI = 4
+    extern __shared__ float out_lds[];
+    float (*out_c)[TILE_N] = reinterpret_cast<float (*)[TILE_N]>(out_lds);
+    int (*out_hi)[TILE_N] = reinterpret_cast<int (*)[TILE_N]>(out_lds + 1 * ROWS * TILE_N);
+    int (*out_lo)[TILE_N] = reinterpret_cast<int (*)[TILE_N]>(out_lds + 2 * ROWS * TILE_N);
+    float (*out_wh)[TILE_N] = reinterpret_cast<float (*)[TILE_N]>(out_lds + 3 * ROWS * TILE_N);
+    float (*out_wl)[TILE_N] = reinterpret_cast<float (*)[TILE_N]>(out_lds + 4 * ROWS * TILE_N);
+    int (*out_ph)[TILE_N] = reinterpret_cast<int (*)[TILE_N]>(out_lds + 5 * ROWS * TILE_N);
+    int (*out_pl)[TILE_N] = reinterpret_cast<int (*)[TILE_N]>(out_lds + 6 * ROWS * TILE_N);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -212,32 +218,37 @@ __global__ __launch_bounds__(NT) void csr_fwd_kernel(
     }
     __syncthreads();
 
-    // one batch row per thread: ROWS consecutive neurons = 16 contiguous bytes per output array
+    // a thread stores 4 consecutive neurons of one batch row: 16 bytes per output array, and the 4
+    // threads of a batch row together one 64-byte run
     const int m0 = blockIdx.x * ROWS;
     const int64_t nm = (int64_t)N * M;
-    for (int o = tid; o < TILE_N; o += NT) {
+    for (int it = tid; it < TILE_N * (ROWS / 4); it += NT_F) {
+        const int o = it / (ROWS / 4), q = it % (ROWS / 4);
         const int n = n0 + o;
-        if (n >= N) break;
-        const int64_t base = (int64_t)n * M + m0;
-        if (vec_out && m0 + ROWS <= M) {
-            *reinterpret_cast<float4 *>(c + base) = make_float4(out_c[0][o], out_c[1][o], out_c[2][o], out_c[3][o]);
-            *reinterpret_cast<int4 *>(argmax + base) = make_int4(out_hi[0][o], out_hi[1][o], out_hi[2][o], out_hi[3][o]);
-            *reinterpret_cast<int4 *>(argmin + base) = make_int4(out_lo[0][o], out_lo[1][o], out_lo[2][o], out_lo[3][o]);
+        if (n >= N) continue;
+        const int r0 = 4 * q;
+        if (m0 + r0 >= M) continue;
+        const int64_t base = (int64_t)n * M + m0 + r0;
+        if (vec_out && m0 + r0 + 4 <= M) {
+            *reinterpret_cast<float4 *>(c + base) = make_float4(out_c[r0][o], out_c[r0 + 1][o], out_c[r0 + 2][o], out_c[r0 + 3][o]);
+            *reinterpret_cast<int4 *>(argmax + base) = make_int4(out_hi[r0][o], out_hi[r0 + 1][o], out_hi[r0 + 2][o], out_hi[r0 + 3][o]);
+            *reinterpret_cast<int4 *>(argmin + base) = make_int4(out_lo[r0][o], out_lo[r0 + 1][o], out_lo[r0 + 2][o], out_lo[r0 + 3][o]);
             if (w_sel) {
-                *reinterpret_cast<float4 *>(w_sel + base) = make_float4(out_wh[0][o], out_wh[1][o], out_wh[2][o], out_wh[3][o]);
-                *reinterpret_cast<float4 *>(w_sel + nm + base) = make_float4(out_wl[0][o], out_wl[1][o], out_wl[2][o], out_wl[3][o]);
+                *reinterpret_cast<float4 *>(w_sel + base) = make_float4(out_wh[r0][o], out_wh[r0 + 1][o], out_wh[r0 + 2][o], out_wh[r0 + 3][o]);
+                *reinterpret_cast<float4 *>(w_sel + nm + base) = make_float4(out_wl[r0][o], out_wl[r0 + 1][o], out_wl[r0 + 2][o], out_wl[r0 + 3][o]);
             }
             if (pos_sel) {
-                *reinterpret_cast<int4 *>(pos_sel + base) = make_int4(out_ph[0][o], out_ph[1][o], out_ph[2][o], out_ph[3][o]);
-                *reinterpret_cast<int4 *>(pos_sel + nm + base) = make_int4(out_pl[0][o], out_pl[1][o], out_pl[2][o], out_pl[3][o]);
+                *reinterpret_cast<int4 *>(pos_sel + base) = make_int4(out_ph[r0][o], out_ph[r0 + 1][o], out_ph[r0 + 2][o], out_ph[r0 + 3][o]);
+                *reinterpret_cast<int4 *>(pos_sel + nm + base) = make_int4(out_pl[r0][o], out_pl[r0 + 1][o], out_pl[r0 + 2][o], out_pl[r0 + 3][o]);
             }
         } else {
-            for (int r = 0; r < ROWS && m0 + r < M; ++r) {
-                c[base + r] = out_c[r][o];
-                argmax[base + r] = out_hi[r][o];
-                argmin[base + r] = out_lo[r][o];
-                if (w_sel) { w_sel[base + r] = out_wh[r][o]; w_sel[nm + base + r] = out_wl[r][o]; }
-                if (pos_sel) { pos_sel[base + r] = out_ph[r][o]; pos_sel[nm + base + r] = out_pl[r][o]; }
+            for (int r = r0; r < r0 + 4 && m0 + r < M; ++r) {
+                const int64_t dst = (int64_t)n * M + m0 + r;
+                c[dst] = out_c[r][o];
+                argmax[dst] = out_hi[r][o];
+                argmin[dst] = out_lo[r][o];
+                if (w_sel) { w_sel[dst] = out_wh[r][o]; w_sel[nm + dst] = out_wl[r][o]; }
+                if (pos_sel) { pos_sel[dst] = out_ph[r][o]; pos_sel[nm + dst] = out_pl[r][o]; }
             }
         }
     }
@@ -378,6 +389,14 @@ __global__ __launch_bounds__(NT) void csr_bwd_val_kernel(
     }
 }
 
+// Lets `kernel` take `bytes` of dynamic LDS (more than the 64 KiB a launch gets by default).
+static int allow_lds(const void *kernel, int bytes)
+{
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) (void)hipGetLastError();
+    return e == hipSuccess;
+}
+
 static int lds_budget_floats(const void *kernel)
 {
     constexpr int kWant = 128 * 1024;
@@ -430,14 +449,19 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
                         ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)w_sel % 16 == 0) &&
                         ((uintptr_t)pos_sel % 16 == 0);
     if (N <= 64) {
-        hipLaunchKernelGGL((csr::csr_fwd_kernel<1>), dim3((unsigned)ceil_div(M, csr::ROWS), 1u), dim3(csr::NT), 0,
+        static const int ok1 = csr::allow_lds((const void *)csr::csr_fwd_kernel<1>, 7 * csr::ROWS * 64 * 4);
+        (void)ok1;
+        hipLaunchKernelGGL((csr::csr_fwd_kernel<1>), dim3((unsigned)ceil_div(M, csr::ROWS), 1u), dim3(csr::NT_F),
+                           (size_t)7 * csr::ROWS * 64 * sizeof(float),
                            st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel, pos_sel, (int)N,
                            (int)K, (int)M, vec_out);
     } else {
         const int64_t gy = ceil_div(N, 256);
         if (gy > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the CSR forward grid");
+        static const int ok4 = csr::allow_lds((const void *)csr::csr_fwd_kernel<4>, 7 * csr::ROWS * 256 * 4);
+        (void)ok4;
         hipLaunchKernelGGL((csr::csr_fwd_kernel<4>), dim3((unsigned)ceil_div(M, csr::ROWS), (unsigned)gy),
-                           dim3(csr::NT), 0, st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel,
+                           dim3(csr::NT_F), (size_t)7 * csr::ROWS * 256 * sizeof(float), st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel,
                            pos_sel, (int)N, (int)K, (int)M, vec_out);
     }
     return check_launch("csr_fwd_kernel");
