@@ -318,7 +318,7 @@ __device__ __forceinline__ void lds_add_sparse(float *addr, float v)
     if (!done) __hip_atomic_fetch_add(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-constexpr int RB = 8;            // CSR rows per val_grad workgroup
+constexpr int RB = 16;           // CSR rows per val_grad workgroup
 constexpr int VAL_CAP = 16384;   // histogram floats per pass (64 KiB)
 
 // val_grad of the entries of RB consecutive CSR rows, from the entry positions recorded by the
