@@ -145,6 +145,37 @@ def test_pruned_dense_weight_with_many_zeros():
     _run_both_layouts(x, w, None, "95% zeros")
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 1), (33, 128, 130), (70, 192, 300), (31, 640, 127), (257, 4096, 129),
+                                   (40, 8192, 260)])
+def test_ragged_batch_and_neurons_on_whole_k_tiles(shape):
+    # K is a multiple of 64, so the (M,K) layout takes the wave-uniform-rows tiling: batch sizes that are no
+    # multiple of its 32 rows, neuron counts that are no multiple of its 128, with and without a split of K
+    N, K, M = shape
+    x, w, _ = random_case(N, K, M, seed=N + M, w_scale=1.0 / K ** 0.5)
+    bias = torch.randn(M, generator=torch.Generator().manual_seed(K))
+    _run_both_layouts(x, w, bias, "whole k tiles %s" % (shape,))
+
+
+def test_aligned_views_with_longer_rows_on_whole_k_tiles():
+    """Aligned 128-k windows of wider x and weight matrices (module splits > 1): row strides exceed K."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(14)
+    N, M, Kfull = 45, 200, 384
+    x = torch.randn(N, Kfull, generator=g); w = torch.randn(M, Kfull, generator=g)
+    xd, wd = x.to(dev), w.to(dev)
+    for k0 in (0, 128, 256):
+        c, amax, amin = capi.fc_forward(xd.narrow(1, k0, 128), wd.narrow(1, k0, 128), capi.W_MK)
+        cv = capi.fc_forward_values(xd.narrow(1, k0, 128), wd.narrow(1, k0, 128), capi.W_MK)
+        torch.cuda.synchronize()
+        want = oracle.forward(x[:, k0:k0 + 128].contiguous().numpy(), w[:, k0:k0 + 128].contiguous().numpy(), oracle.W_MK)
+        assert_bits_equal(c.cpu().numpy(), want[0], "window %d c" % k0)
+        assert_index_equal(amax.cpu().numpy(), want[1], "window %d argmax" % k0)
+        assert_index_equal(amin.cpu().numpy(), want[2], "window %d argmin" % k0)
+        assert_bits_equal(cv.cpu().numpy(), want[0], "window %d values-only c" % k0)
+
+
 def test_strided_rows_and_unaligned_views():
     from mamtorch_amd import capi
 
