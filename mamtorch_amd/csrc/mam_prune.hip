@@ -111,30 +111,36 @@ __global__ __launch_bounds__(NT) void count_kernel(const float *__restrict__ w, 
     if (m == 0 && lane == 0) crow[0] = 0;
 }
 
-// crow[1..M] holds row counts on entry and inclusive prefix sums on exit.  One workgroup.
+// crow[1..M] holds row counts on entry and inclusive prefix sums on exit.  One workgroup: a thread
+// takes a run of consecutive rows, waves scan their threads' sums with shuffles, one more step
+// chains the 16 waves.
 __global__ __launch_bounds__(1024) void scan_kernel(int64_t *__restrict__ crow, int M)
 {
-    __shared__ int64_t partial[1024];
-    __shared__ int64_t carry;
-    const int tid = threadIdx.x;
-    if (tid == 0) carry = 0;
+    __shared__ int64_t wave_total[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int per = (M + 1023) / 1024;
+    const int first = tid * per;
+    int64_t sum = 0;
+    for (int j = 0; j < per; ++j) {
+        const int i = first + j;
+        if (i < M) sum += crow[i + 1];
+    }
+    int64_t incl = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int64_t t = __shfl_up(incl, off);
+        if (lane >= off) incl += t;
+    }
+    if (lane == 63) wave_total[wave] = incl;
     __syncthreads();
-    for (int base = 0; base < M; base += 1024) {
-        const int i = base + tid;
-        const int64_t v = i < M ? crow[i + 1] : 0;
-        partial[tid] = v;
-        __syncthreads();
-        for (int off = 1; off < 1024; off <<= 1) {
-            const int64_t add = tid >= off ? partial[tid - off] : 0;
-            __syncthreads();
-            partial[tid] += add;
-            __syncthreads();
+    int64_t run = incl - sum;
+    for (int w2 = 0; w2 < wave; ++w2) run += wave_total[w2];
+    for (int j = 0; j < per; ++j) {
+        const int i = first + j;
+        if (i < M) {
+            run += crow[i + 1];
+            crow[i + 1] = run;
         }
-        const int64_t before = carry;
-        if (i < M) crow[i + 1] = before + partial[tid];
-        __syncthreads();
-        if (tid == 1023) carry = before + partial[1023];
-        __syncthreads();
     }
 }
 
