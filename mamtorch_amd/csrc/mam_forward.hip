@@ -157,26 +157,43 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
 }
 
 // Cooperative resolve of the 64 outputs held by one wave (fast layouts only: (M,K) weight,
-// 16-byte aligned rows, K a multiple of G).  The cost of resolving is cache-line lookups, so the
-// G/4 lanes of a task each fetch one 16-byte chunk of x and of w: a task touches one contiguous
-// G*4-byte segment per operand instead of G/4 lanes each touching G/4 segments.  128 tasks
-// (64 outputs x {max, min}) are processed 64/(G/4) per round.
+// 16-byte aligned rows, K a multiple of G).  The cost of resolving is cache-line lookups plus the
+// instructions around them, so the G/4 lanes of a task each fetch one 16-byte chunk of x and of w
+// (a task touches one contiguous G*4-byte segment per operand), the lanes of a task agree on the
+// first match with two DPP min steps (no LDS permutes), only the winning lane writes the task's
+// result to LDS, and in a second pass lane s stores output s: whole-wave stores, contiguous where
+// consecutive slots are consecutive neurons.  128 tasks (64 outputs x {max, min}), 64/(G/4) per
+// round.
 //   vals : LDS, [2][64]  running max, running min of the wave's outputs
 //   grps : LDS, [2][64]  absolute group id of the max, of the min
+//   res  : LDS, [6][64]  scratch of this wave: value, index, weight of the max and of the min
 //   nm_of(slot, n, m, valid): output coordinates of slot 0..63 (clamped into range when !valid)
 constexpr int LPT = G / 4;             // lanes per task
 constexpr int TPR = 64 / LPT;          // tasks per round
 constexpr int RES_ROUNDS = 128 / TPR;
+constexpr int RES_WORDS = 6 * 64;      // LDS words of `res` per wave
+static_assert(LPT == 4, "the lane exchange below is written for 4 lanes per task");
+
+__device__ __forceinline__ int quad_min(int v)
+{
+    // minimum over the 4 lanes of a quad: neighbours (quad_perm [1,0,3,2]), then pairs ([2,3,0,1])
+    int o = __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, true);
+    v = o < v ? o : v;
+    o = __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, true);
+    return o < v ? o : v;
+}
 
 template <class NM>
-__device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps,
+__device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps, float *res,
                                              int lane, NM nm_of)
 {
-    // Two passes over the rounds, both unrolled: every load of every round first (stores
-    // between them would pin the loads in program order), then the stores.
-    float r_sum[RES_ROUNDS], r_wmax[RES_ROUNDS], r_wmin[RES_ROUNDS];
-    int r_imax[RES_ROUNDS], r_imin[RES_ROUNDS];
-    int64_t r_out[RES_ROUNDS];
+    float *res_v = res;                                    // [2][64]
+    int *res_i = reinterpret_cast<int *>(res + 128);        // [2][64]
+    float *res_w = res + 256;                               // [2][64]
+    // every load of every round first, then the matching
+    float4 xa[RES_ROUNDS], wa[RES_ROUNDS];
+    float target[RES_ROUNDS];
+    int grp[RES_ROUNDS];
 #pragma unroll
     for (int r = 0; r < RES_ROUNDS; ++r) {
         const int task = r * TPR + lane / LPT;
@@ -184,53 +201,48 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
         int n, m;
         bool valid;
         nm_of(slot, n, m, valid);
-        const float target = vals[ext * 64 + slot];
-        const int g = grps[ext * 64 + slot];
-        const int kb = g * G + sub * 4;
-        const float4 xa = *reinterpret_cast<const float4 *>(p.x + (int64_t)n * p.ldx + kb);
-        const float4 wa = *reinterpret_cast<const float4 *>(p.w + (int64_t)m * p.ldw + kb);
-        const float p0 = xa.x * wa.x, p1 = xa.y * wa.y, p2 = xa.z * wa.z, p3 = xa.w * wa.w;
-        // position within the group of this lane's first match (lowest wins), 255 = none
-        int key = 255;
-        float val = target;
-        float wsel = wa.x;         // fallback: the first weight of the group (only lane sub 0 can keep it)
-        if (p3 == target) { key = sub * 4 + 3; val = p3; wsel = wa.w; }
-        if (p2 == target) { key = sub * 4 + 2; val = p2; wsel = wa.z; }
-        if (p1 == target) { key = sub * 4 + 1; val = p1; wsel = wa.y; }
-        if (p0 == target) { key = sub * 4 + 0; val = p0; wsel = wa.x; }
-        if (key == 255 && sub == 0) key = 254;   // no match anywhere: lane 0's fallback wins the reduce
-#pragma unroll
-        for (int off = 1; off < LPT; off <<= 1) {
-            const int okey = __shfl_xor(key, off);
-            const float oval = __shfl_xor(val, off);
-            const float owsel = __shfl_xor(wsel, off);
-            if (okey < key) { key = okey; val = oval; wsel = owsel; }
-        }
-        if (key >= 254) key = 0;   // no product equals the extreme (NaN operands): first of the group
-        const int idx = g * G + key;
-        // lanes of the max task and of the min task of one output are LPT apart
-        const float val_min = __shfl_xor(val, LPT);
-        float sum = val + val_min;
-        if (p.bias) sum = sum + p.bias[m];
-        r_sum[r] = sum;
-        r_imax[r] = idx;
-        r_imin[r] = __shfl_xor(idx, LPT);
-        r_wmax[r] = wsel;
-        r_wmin[r] = __shfl_xor(wsel, LPT);
-        r_out[r] = (ext == 0 && sub == 0 && valid) ? (int64_t)n * p.M + m : (int64_t)-1;
+        target[r] = vals[ext * 64 + slot];
+        grp[r] = grps[ext * 64 + slot];
+        const int kb = grp[r] * G + sub * 4;
+        xa[r] = *reinterpret_cast<const float4 *>(p.x + (int64_t)n * p.ldx + kb);
+        wa[r] = *reinterpret_cast<const float4 *>(p.w + (int64_t)m * p.ldw + kb);
     }
-    const int64_t nm = (int64_t)p.N * p.M;
 #pragma unroll
     for (int r = 0; r < RES_ROUNDS; ++r) {
-        const int64_t o = r_out[r];
-        if (o >= 0) {
-            p.c[o] = r_sum[r];
-            p.argmax[o] = r_imax[r];
-            p.argmin[o] = r_imin[r];
-            if (p.wsel) {
-                p.wsel[o] = r_wmax[r];
-                p.wsel[nm + o] = r_wmin[r];
-            }
+        const int task = r * TPR + lane / LPT;
+        const int slot = task >> 1, ext = task & 1, sub = lane % LPT;
+        const float p0 = xa[r].x * wa[r].x, p1 = xa[r].y * wa[r].y, p2 = xa[r].z * wa[r].z, p3 = xa[r].w * wa[r].w;
+        // position within the group of this lane's first match (lowest wins), 255 = none
+        int key = 255;
+        float val = target[r];
+        float wsel = wa[r].x;      // kept only by the fallback below
+        if (p3 == target[r]) { key = sub * 4 + 3; val = p3; wsel = wa[r].w; }
+        if (p2 == target[r]) { key = sub * 4 + 2; val = p2; wsel = wa[r].z; }
+        if (p1 == target[r]) { key = sub * 4 + 1; val = p1; wsel = wa[r].y; }
+        if (p0 == target[r]) { key = sub * 4 + 0; val = p0; wsel = wa[r].x; }
+        const int best = quad_min(key);
+        // no product equals the extreme (NaN operands): the first k of the group, from lane 0
+        const bool fallback = best == 255 && sub == 0;
+        if ((key == best && key != 255) || fallback) {
+            res_v[ext * 64 + slot] = val;
+            res_i[ext * 64 + slot] = grp[r] * G + (fallback ? 0 : key);
+            res_w[ext * 64 + slot] = wsel;
+        }
+    }
+    // lane s finishes output s
+    int n, m;
+    bool valid;
+    nm_of(lane, n, m, valid);
+    float sum = res_v[lane] + res_v[64 + lane];
+    if (p.bias) sum = sum + p.bias[m];
+    if (valid) {
+        const int64_t o = (int64_t)n * p.M + m;
+        p.c[o] = sum;
+        p.argmax[o] = res_i[lane];
+        p.argmin[o] = res_i[64 + lane];
+        if (p.wsel) {
+            p.wsel[o] = res_w[lane];
+            p.wsel[(int64_t)p.N * p.M + o] = res_w[64 + lane];
         }
     }
 }
@@ -531,6 +543,8 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
         const int lane = tid & 63;
         float *vals = tile_a + wave * (TJ * 2 * 64);
         int *grps = reinterpret_cast<int *>(tile_b) + wave * (TJ * 2 * 64);
+        static_assert((NT / 64) * (TJ * 2 * 64 + RES_WORDS) <= TILE_FLOATS, "resolve scratch does not fit");
+        float *res = tile_a + (NT / 64) * (TJ * 2 * 64) + wave * RES_WORDS;
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
             __syncthreads();
@@ -545,7 +559,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 #pragma unroll 1
             for (int j = 0; j < TJ; ++j) {
                 const int nbase = row0 + 16 * i + 4 * wave, mbase = col0 + 16 * j;
-                resolve_wave(p, vals + j * 128, grps + j * 128, lane,
+                resolve_wave(p, vals + j * 128, grps + j * 128, res, lane,
                              [&](int slot, int &n, int &m, bool &valid) {
                                  n = nbase + (slot >> 4);
                                  m = mbase + (slot & 15);
@@ -610,6 +624,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
     // one 16-neuron range run back to back on one XCD keeps those 16 weight rows in that L2.
     __shared__ float vals_s[4][2][64];
     __shared__ int grps_s[4][2][64];
+    __shared__ float res_s[4][RES_WORDS];
     const int64_t nm = (int64_t)p.N * p.M;
     const int patches_n = (p.N + 15) / 16;
     const int logical = xcd_remap(blockIdx.x, gridDim.x);
@@ -653,7 +668,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
         grps_s[wave][1][lane] = gmin;
         __syncthreads();
         const int nbase = pn * 16 + 4 * wave, mbase = pm * 16;
-        resolve_wave(p, &vals_s[wave][0][0], &grps_s[wave][0][0], lane,
+        resolve_wave(p, &vals_s[wave][0][0], &grps_s[wave][0][0], &res_s[wave][0], lane,
                      [&](int slot, int &n, int &m, bool &valid) {
                          n = nbase + (slot >> 4);
                          m = mbase + (slot & 15);
@@ -856,6 +871,8 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
         // and resolves it set by set; the 64 outputs of a set share their x row.
         float *vals = tile_a + wave * (sx::TJ * 128);
         int *grps = reinterpret_cast<int *>(tile_b) + wave * (sx::TJ * 128);
+        static_assert((sx::NT / 64) * (sx::TJ * 128 + RES_WORDS) <= sx::TILE_FLOATS, "resolve scratch does not fit");
+        float *res = tile_a + (sx::NT / 64) * (sx::TJ * 128) + wave * RES_WORDS;
 #pragma unroll
         for (int i = 0; i < sx::TI; ++i) {
             __syncthreads();
@@ -871,7 +888,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 #pragma unroll 1
             for (int j = 0; j < sx::TJ; ++j) {
                 const int mbase = col0 + 64 * j;
-                resolve_wave(p, vals + j * 128, grps + j * 128, lane,
+                resolve_wave(p, vals + j * 128, grps + j * 128, res, lane,
                              [&](int slot, int &n, int &m, bool &valid) {
                                  n = nrow;
                                  m = mbase + slot;
