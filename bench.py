@@ -40,7 +40,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the headline shape from the FETCH_SIZE / WRITE_SIZE counters, each scaled
 # by what the same counter reads for the plain 64 MiB copy made before the warm-up
 # (profiles/hbm_traffic_headline_n256_k4096_m4096.md)
-FORWARD_TRAFFIC_BYTES = {"mam_fwd_sx_kernel": 138.5e6, "mam_fwd_merge_kernel": 141.6e6}
+FORWARD_TRAFFIC_BYTES = {"mam_fwd_sx_kernel": 140.1e6, "mam_fwd_merge_kernel": 133.5e6}
 BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 102.4e6}
 
 WORKLOADS = ("headline", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
