@@ -64,9 +64,11 @@ class Layer:
         if want_backward:
             self.xg = torch.empty((N, K), dtype=torch.float32, device=dev)
             self.wg = torch.empty((M, K), dtype=torch.float32, device=dev)
-            self.wsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)  # forward -> backward
+            # selected weights and inputs, forward -> backward
+            self.wsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)
+            self.xsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)
         else:
-            self.wsel = None
+            self.wsel = self.xsel = None
         if want_count:
             self.max_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
             self.min_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
@@ -86,14 +88,15 @@ class Layer:
                                                 N, K, M, P(self.ws), self.ws_bytes, self.sp)
         else:
             rc = self.lib.mam_fc_forward(P(self.x), K, P(self.w), K, self.capi.W_MK, None, P(self.c),
-                                         P(self.amax), P(self.amin), P(self.wsel), N, K, M, P(self.ws),
+                                         P(self.amax), P(self.amin), P(self.wsel), P(self.xsel), N, K, M, P(self.ws),
                                          self.ws_bytes, self.sp)
         assert rc == 0, self.lib.mam_last_error()
 
     def backward(self):
         P, N, K, M = self._p, self.N, self.K, self.M
         rc = self.lib.mam_fc_backward(P(self.x), K, P(self.w), K, self.capi.W_MK, P(self.g), P(self.amax),
-                                      P(self.amin), P(self.wsel), P(self.xg), P(self.wg), N, K, M, self.sp)
+                                      P(self.amin), P(self.wsel), P(self.xsel), P(self.xg), P(self.wg), N, K, M,
+                                      self.sp)
         assert rc == 0, self.lib.mam_last_error()
 
     def count(self):

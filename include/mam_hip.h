@@ -62,11 +62,13 @@ const char *mam_last_error(void);
  * `workspace` may be NULL when mam_fc_forward_workspace() returns 0.
  * `w_sel` (optional, may be NULL): (2, N, M) fp32 contiguous; receives w[argmax[n,m], m] in plane 0 and
  * w[argmin[n,m], m] in plane 1.  Handing it to mam_fc_backward spares that call 2*N*M random reads of w.
+ * `x_sel` (optional, may be NULL): the same for the inputs, x[n, argmax[n,m]] and x[n, argmin[n,m]]; it
+ * spares mam_fc_backward the 2*N*M random reads of x behind w_grad.
  */
 size_t mam_fc_forward_workspace(int64_t N, int64_t K, int64_t M);
 int mam_fc_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                    const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel,
-                   int64_t N, int64_t K, int64_t M,
+                   float *x_sel, int64_t N, int64_t K, int64_t M,
                    void *workspace, size_t workspace_bytes, void *stream);
 
 /*
@@ -85,14 +87,15 @@ int mam_fc_forward_values(const float *x, int64_t ldx, const float *w, int64_t l
  *   w_grad[k,m] = sum_n grad[n,m] * x[n,k] * (same)          (argmax==argmin counts twice)
  * x_grad (N,K) and w_grad (layout and shape of w, contiguous) are fully overwritten.
  * Either output pointer may be NULL to skip it.  grad/argmax/argmin are (N,M) contiguous.
- * `w_sel` (optional, may be NULL) is the (2, N, M) array written by mam_fc_forward for the same inputs.
+ * `w_sel` and `x_sel` (optional, each may be NULL) are the (2, N, M) arrays written by mam_fc_forward for
+ * the same inputs; x_grad uses w_sel, w_grad uses x_sel, and whichever is NULL is gathered from w / x.
  * Replaces fullyconnected_backward_cuda
  * (mamtorch/kernel/v4/csrc/cuda/fullyconnected_backward.cu:80-135, kernel :24-78; v1 identical).
  * Indices outside [0,K) make the call's result undefined for that output only (they are skipped).
  */
 int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                     const float *grad, const int32_t *argmax, const int32_t *argmin, const float *w_sel,
-                    float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, void *stream);
+                    const float *x_sel, float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, void *stream);
 
 /*
  * Selection-count accumulation for pruning: adds this batch's picks into (M,K) int32 counters

@@ -47,12 +47,12 @@ def lib():
             fn = getattr(l, name)
             fn.restype = _size
             fn.argtypes = [_i64, _i64, _i64]
-        l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
-                                     _i64, _ptr, _size, _ptr]
+        l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
+                                     _i64, _i64, _ptr, _size, _ptr]
         l.mam_fc_forward_values.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _i64, _i64, _i64,
                                             _ptr, _size, _ptr]
-        l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
-                                      _i64, _i64, _ptr]
+        l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                      _i64, _i64, _i64, _ptr]
         l.mam_selection_count.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr]
         l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                          _i64, _i64, _i64, _i64, _ptr, _size, _ptr]
@@ -98,9 +98,9 @@ def _ld(t):
     return t.stride(0) if t.size(0) > 1 else max(t.size(1), 1)
 
 
-def fc_forward(x, w, layout=W_KM, bias=None, workspace=None, w_sel=None):
+def fc_forward(x, w, layout=W_KM, bias=None, workspace=None, w_sel=None, x_sel=None):
     """-> (c, argmax, argmin) on x.device.  ``workspace`` (uint8 tensor) is allocated if None.
-    ``w_sel``: optional (2, N, M) fp32 tensor that receives the selected weights."""
+    ``w_sel`` / ``x_sel``: optional (2, N, M) fp32 tensors that receive the selected weights / inputs."""
     l = lib()
     N, K, M = _dims(x, w, layout)
     c = torch.empty((N, M), dtype=torch.float32, device=x.device)
@@ -111,7 +111,7 @@ def fc_forward(x, w, layout=W_KM, bias=None, workspace=None, w_sel=None):
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         _check(l.mam_fc_forward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(bias), _p(c), _p(amax), _p(amin),
-                                _p(w_sel), N, K, M, _p(workspace), 0 if workspace is None else workspace.numel(),
+                                _p(w_sel), _p(x_sel), N, K, M, _p(workspace), 0 if workspace is None else workspace.numel(),
                                 _stream(x)))
     return c, amax, amin
 
@@ -130,7 +130,7 @@ def fc_forward_values(x, w, layout=W_KM, bias=None, workspace=None):
     return c
 
 
-def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=True, w_sel=None):
+def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=True, w_sel=None, x_sel=None):
     """-> (x_grad or None, w_grad or None); w_grad has the shape and layout of w."""
     l = lib()
     N, K, M = _dims(x, w, layout)
@@ -138,7 +138,7 @@ def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=Tru
     wg = torch.empty(tuple(w.shape), dtype=torch.float32, device=x.device) if want_w else None
     with torch.cuda.device(x.device):
         _check(l.mam_fc_backward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(grad), _p(argmax), _p(argmin),
-                                 _p(w_sel), _p(xg), _p(wg), N, K, M, _stream(x)))
+                                 _p(w_sel), _p(x_sel), _p(xg), _p(wg), N, K, M, _stream(x)))
     return xg, wg
 
 

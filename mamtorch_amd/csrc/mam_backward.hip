@@ -172,8 +172,8 @@ template <int LAYOUT>
 __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    float *__restrict__ w_grad, int N, int K, int M, int log2r, int kc, int vec_out, int mtiles,
-    int tiles_per_wg)
+    const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
+    int kc, int vec_out, int mtiles, int tiles_per_wg)
 {
     extern __shared__ float hist[];
     const int tid = threadIdx.x;
@@ -187,6 +187,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
     // this thread's first item of a slab: row n_first, neurons m0 + r_first .. +3
     const int n_first = tid / qpr, r_first = (tid - n_first * qpr) * 4;
     float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 s1 = g, s2 = g;      // selected inputs handed over by the forward, if any
     int4 i1 = make_int4(-1, -1, -1, -1), i2 = make_int4(-1, -1, -1, -1);
     bool have = false;
     auto load_first = [&](int m0) {
@@ -196,6 +197,10 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
             g = *reinterpret_cast<const float4 *>(grad + o);
             i1 = *reinterpret_cast<const int4 *>(argmax + o);
             i2 = *reinterpret_cast<const int4 *>(argmin + o);
+            if (x_sel) {
+                s1 = *reinterpret_cast<const float4 *>(x_sel + o);
+                s2 = *reinterpret_cast<const float4 *>(x_sel + nm + o);
+            }
         }
     };
     if (first < mtiles) load_first(first * R);
@@ -205,8 +210,8 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
         if (mt >= mtiles) break;
         const int m0 = mt * R;
         const int rn = (M - m0) < R ? (M - m0) : R;
-        float x1[4], x2[4];
-        if (have) gather_quad(x + (int64_t)n_first * ldx + k0, i1, i2, k0, kn, x1, x2);
+        float x1[4] = {s1.x, s1.y, s1.z, s1.w}, x2[4] = {s2.x, s2.y, s2.z, s2.w};
+        if (have && !x_sel) gather_quad(x + (int64_t)n_first * ldx + k0, i1, i2, k0, kn, x1, x2);
         for (int i = tid * 4; i < R * kc; i += NT_W * 4)
             *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
@@ -219,7 +224,14 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
             const int4 j1 = *reinterpret_cast<const int4 *>(argmax + o);
             const int4 j2 = *reinterpret_cast<const int4 *>(argmin + o);
             float y1[4], y2[4];
-            gather_quad(x + (int64_t)n * ldx + k0, j1, j2, k0, kn, y1, y2);
+            if (x_sel) {
+                const float4 t1 = *reinterpret_cast<const float4 *>(x_sel + o);
+                const float4 t2 = *reinterpret_cast<const float4 *>(x_sel + nm + o);
+                y1[0] = t1.x; y1[1] = t1.y; y1[2] = t1.z; y1[3] = t1.w;
+                y2[0] = t2.x; y2[1] = t2.y; y2[2] = t2.z; y2[3] = t2.w;
+            } else {
+                gather_quad(x + (int64_t)n * ldx + k0, j1, j2, k0, kn, y1, y2);
+            }
             scatter_quad<LAYOUT>(hist, gg, j1, j2, y1, y2, r0, k0, kn, kc, log2r);
         }
         __syncthreads();
@@ -234,7 +246,8 @@ template <int LAYOUT>
 __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    float *__restrict__ w_grad, int N, int K, int M, int log2r, int kc, int vec_out)
+    const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
+    int kc, int vec_out)
 {
     extern __shared__ float hist[];
     const int tid = threadIdx.x;
@@ -257,9 +270,11 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
         const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
         const float *xr = x + (int64_t)n * ldx + k0;
         if ((unsigned)a1 < (unsigned)kn)
-            lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r], xr[a1] * g);
+            lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r],
+                           (x_sel ? x_sel[o] : xr[a1]) * g);
         if ((unsigned)a2 < (unsigned)kn)
-            lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r], xr[a2] * g);
+            lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r],
+                           (x_sel ? x_sel[nm + o] : xr[a2]) * g);
     }
     __syncthreads();
     store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out);
@@ -278,7 +293,7 @@ static int lds_budget_floats(const void *kernel)
 
 template <int LAYOUT>
 static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ldw, const float *grad,
-                         const int32_t *argmax, const int32_t *argmin, const float *w_sel,
+                         const int32_t *argmax, const int32_t *argmin, const float *w_sel, const float *x_sel,
                          float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
 {
     int rc = MAM_OK;
@@ -306,7 +321,7 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         if (ktiles > 65535) return fail(MAM_ERR_UNSUPPORTED, "K too large for the w_grad grid");
         const int vec_out = (K % 4 == 0) && ((uintptr_t)w_grad % 16 == 0);
         const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
-                           ((uintptr_t)argmin % 16 == 0);
+                           ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)x_sel % 16 == 0) && (N * M % 4 == 0);
         if (vec_in) {
             // slabs per workgroup: enough workgroups for two per CU, the rest goes into pipelining
             int tpw = (int)(mtiles * ktiles / (2 * kNumCU));
@@ -314,12 +329,12 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
             if (tpw > 8) tpw = 8;
             hipLaunchKernelGGL((mam_bwd_w_vec_kernel<LAYOUT>),
                                dim3((unsigned)ceil_div(mtiles, tpw), (unsigned)ktiles), dim3(NT_W),
-                               (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax, argmin, w_grad,
-                               (int)N, (int)K, (int)M, log2r, kc, vec_out, (int)mtiles, tpw);
+                               (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax, argmin, x_sel, N * M,
+                               w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out, (int)mtiles, tpw);
         } else {
             hipLaunchKernelGGL((mam_bwd_w_kernel<LAYOUT>), dim3((unsigned)mtiles, (unsigned)ktiles),
                                dim3(NT_W), (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax,
-                               argmin, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out);
+                               argmin, x_sel, N * M, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out);
         }
         rc = check_launch("mam_bwd_w_kernel");
     }
@@ -343,8 +358,8 @@ int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t
 
 extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                                const float *grad, const int32_t *argmax, const int32_t *argmin,
-                               const float *w_sel, float *x_grad, float *w_grad, int64_t N, int64_t K,
-                               int64_t M, void *stream)
+                               const float *w_sel, const float *x_sel, float *x_grad, float *w_grad,
+                               int64_t N, int64_t K, int64_t M, void *stream)
 {
     using namespace mam;
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
@@ -364,6 +379,6 @@ extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int6
     if (ldx < K || ldw < (w_layout == MAM_W_MK ? K : M))
         return fail(MAM_ERR_INVALID_ARGUMENT, "leading dimension smaller than the row length");
     if (w_layout == MAM_W_MK)
-        return bwd::launch_layout<MAM_W_MK>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_grad, w_grad, N, K, M, st);
-    return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_grad, w_grad, N, K, M, st);
+        return bwd::launch_layout<MAM_W_MK>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, x_grad, w_grad, N, K, M, st);
+    return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, x_grad, w_grad, N, K, M, st);
 }

@@ -62,6 +62,7 @@ struct Params {
     int32_t *argmax;
     int32_t *argmin;
     float *wsel;      // optional [2][N*M]: the selected weights w[argmax], w[argmin] (for the backward)
+    float *xsel;      // optional [2][N*M]: the selected inputs x[argmax], x[argmin] (for the backward)
     float *part;      // split-K partials: [split][3 or 2][N*M]: max, min, (group ids packed 16:16)
     int N, K, M;
     int tiles_n, tiles_m, splits, k_per_split;
@@ -75,7 +76,7 @@ struct Params {
 // G operands of each side are fetched with 16-byte loads when the layout allows it.
 template <int LAYOUT>
 __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, float target,
-                                        float &val, int &idx, float &wsel)
+                                        float &val, int &idx, float &wsel, float &xsel)
 {
     const int kb = g * G;
     const int klast = p.K - 1;
@@ -83,6 +84,7 @@ __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, fl
     val = target;
     const float *xr = p.x + (int64_t)n * p.ldx;
     wsel = load_w<LAYOUT>(p.w, p.ldw, idx, m);
+    xsel = xr[idx];
     float xv[G], wv[G];
     const bool whole = kb + G <= p.K;
     if (whole && p.vec_x) {
@@ -110,7 +112,7 @@ __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, fl
 #pragma unroll
     for (int kk = G - 1; kk >= 0; --kk) {
         const float prod = xv[kk] * wv[kk];
-        if (prod == target) { idx = (kb + kk) < klast ? (kb + kk) : klast; val = prod; wsel = wv[kk]; }
+        if (prod == target) { idx = (kb + kk) < klast ? (kb + kk) : klast; val = prod; wsel = wv[kk]; xsel = xv[kk]; }
     }
 }
 
@@ -134,10 +136,10 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
 {
     float hi = vmax, lo = vmin;
     int ih = 0, il = 0;
-    float wh = 0.0f, wl = 0.0f;
+    float wh = 0.0f, wl = 0.0f, xh = 0.0f, xl = 0.0f;
     if (ARGS) {
-        resolve<LAYOUT>(p, n, m, gmax, vmax, hi, ih, wh);
-        resolve<LAYOUT>(p, n, m, gmin, vmin, lo, il, wl);
+        resolve<LAYOUT>(p, n, m, gmax, vmax, hi, ih, wh, xh);
+        resolve<LAYOUT>(p, n, m, gmin, vmin, lo, il, wl, xl);
     } else {
         if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m);
         if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m);
@@ -153,6 +155,10 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
             p.wsel[o] = wh;
             p.wsel[(int64_t)p.N * p.M + o] = wl;
         }
+        if (p.xsel) {
+            p.xsel[o] = xh;
+            p.xsel[(int64_t)p.N * p.M + o] = xl;
+        }
     }
 }
 
@@ -166,12 +172,12 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
 // round.
 //   vals : LDS, [2][64]  running max, running min of the wave's outputs
 //   grps : LDS, [2][64]  absolute group id of the max, of the min
-//   res  : LDS, [6][64]  scratch of this wave: value, index, weight of the max and of the min
+//   res  : LDS, [8][64]  scratch of this wave: value, index, weight, input of the max and of the min
 //   nm_of(slot, n, m, valid): output coordinates of slot 0..63 (clamped into range when !valid)
 constexpr int LPT = G / 4;             // lanes per task
 constexpr int TPR = 64 / LPT;          // tasks per round
 constexpr int RES_ROUNDS = 128 / TPR;
-constexpr int RES_WORDS = 6 * 64;      // LDS words of `res` per wave
+constexpr int RES_WORDS = 8 * 64;      // LDS words of `res` per wave
 static_assert(LPT == 4, "the lane exchange below is written for 4 lanes per task");
 
 __device__ __forceinline__ int quad_min(int v)
@@ -190,6 +196,7 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
     float *res_v = res;                                    // [2][64]
     int *res_i = reinterpret_cast<int *>(res + 128);        // [2][64]
     float *res_w = res + 256;                               // [2][64]
+    float *res_x = res + 384;                               // [2][64]
     // every load of every round first, then the matching
     float4 xa[RES_ROUNDS], wa[RES_ROUNDS];
     float target[RES_ROUNDS];
@@ -214,19 +221,20 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
         const float p0 = xa[r].x * wa[r].x, p1 = xa[r].y * wa[r].y, p2 = xa[r].z * wa[r].z, p3 = xa[r].w * wa[r].w;
         // position within the group of this lane's first match (lowest wins), 255 = none
         int key = 255;
-        float val = target[r];
-        float wsel = wa[r].x;      // kept only by the fallback below
-        if (p3 == target[r]) { key = sub * 4 + 3; val = p3; wsel = wa[r].w; }
-        if (p2 == target[r]) { key = sub * 4 + 2; val = p2; wsel = wa[r].z; }
-        if (p1 == target[r]) { key = sub * 4 + 1; val = p1; wsel = wa[r].y; }
-        if (p0 == target[r]) { key = sub * 4 + 0; val = p0; wsel = wa[r].x; }
+        float wsel = wa[r].x, xsel = xa[r].x;      // kept only by the fallback below
+        if (p3 == target[r]) { key = sub * 4 + 3; wsel = wa[r].w; xsel = xa[r].w; }
+        if (p2 == target[r]) { key = sub * 4 + 2; wsel = wa[r].z; xsel = xa[r].z; }
+        if (p1 == target[r]) { key = sub * 4 + 1; wsel = wa[r].y; xsel = xa[r].y; }
+        if (p0 == target[r]) { key = sub * 4 + 0; wsel = wa[r].x; xsel = xa[r].x; }
         const int best = quad_min(key);
         // no product equals the extreme (NaN operands): the first k of the group, from lane 0
         const bool fallback = best == 255 && sub == 0;
         if ((key == best && key != 255) || fallback) {
-            res_v[ext * 64 + slot] = val;
+            // the value is recomputed from the selected operands (the sign of a zero follows them)
+            res_v[ext * 64 + slot] = fallback ? target[r] : xsel * wsel;
             res_i[ext * 64 + slot] = grp[r] * G + (fallback ? 0 : key);
             res_w[ext * 64 + slot] = wsel;
+            res_x[ext * 64 + slot] = xsel;
         }
     }
     // lane s finishes output s
@@ -243,6 +251,10 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
         if (p.wsel) {
             p.wsel[o] = res_w[lane];
             p.wsel[(int64_t)p.N * p.M + o] = res_w[64 + lane];
+        }
+        if (p.xsel) {
+            p.xsel[o] = res_x[lane];
+            p.xsel[(int64_t)p.N * p.M + o] = res_x[64 + lane];
         }
     }
 }
@@ -961,8 +973,8 @@ static size_t workspace_bytes(int64_t N, int64_t K, int64_t M, bool args)
 
 template <bool ARGS>
 static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
-                  const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, int64_t N,
-                  int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream)
+                  const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel,
+                  int64_t N, int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream)
 {
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
     if (w_layout != MAM_W_KM && w_layout != MAM_W_MK)
@@ -978,7 +990,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
 
     Params p;
     p.x = x; p.ldx = ldx; p.w = w; p.ldw = ldw; p.bias = bias;
-    p.c = c; p.argmax = argmax; p.argmin = argmin; p.wsel = w_sel;
+    p.c = c; p.argmax = argmax; p.argmin = argmin; p.wsel = w_sel; p.xsel = x_sel;
     p.N = (int)N; p.K = (int)K; p.M = (int)M;
     p.vec_x = (ldx % 4 == 0) && ((uintptr_t)x % 16 == 0);
     p.vec_w = (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0);
@@ -1054,10 +1066,10 @@ extern "C" size_t mam_fc_forward_values_workspace(int64_t N, int64_t K, int64_t 
 
 extern "C" int mam_fc_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                               const float *bias, float *c, int32_t *argmax, int32_t *argmin,
-                              float *w_sel, int64_t N, int64_t K, int64_t M, void *workspace,
-                              size_t workspace_bytes, void *stream)
+                              float *w_sel, float *x_sel, int64_t N, int64_t K, int64_t M,
+                              void *workspace, size_t workspace_bytes, void *stream)
 {
-    return mam::fwd::launch<true>(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, N, K, M,
+    return mam::fwd::launch<true>(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, x_sel, N, K, M,
                                   workspace, workspace_bytes, stream);
 }
 
@@ -1065,6 +1077,6 @@ extern "C" int mam_fc_forward_values(const float *x, int64_t ldx, const float *w
                                      int w_layout, const float *bias, float *c, int64_t N, int64_t K,
                                      int64_t M, void *workspace, size_t workspace_bytes, void *stream)
 {
-    return mam::fwd::launch<false>(x, ldx, w, ldw, w_layout, bias, c, nullptr, nullptr, nullptr, N, K, M,
+    return mam::fwd::launch<false>(x, ldx, w, ldw, w_layout, bias, c, nullptr, nullptr, nullptr, nullptr, N, K, M,
                                    workspace, workspace_bytes, stream);
 }

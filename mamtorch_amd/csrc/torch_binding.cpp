@@ -97,18 +97,21 @@ const float *bias_ptr(const c10::optional<at::Tensor> &bias)
 }
 
 std::vector<at::Tensor> forward_impl(const at::Tensor &a, const at::Tensor &w, int layout,
-                                     const c10::optional<at::Tensor> &bias, bool want_w_sel)
+                                     const c10::optional<at::Tensor> &bias, bool with_sel, bool hand_over)
 {
     const FwdShape s = check_forward(a, w, layout, bias);
     const c10::DeviceGuard guard(a.device());
     auto c = at::empty({s.N, s.M}, a.options());
     auto argmax = at::empty({s.N, s.M}, a.options().dtype(at::kInt));
     auto argmin = at::empty({s.N, s.M}, a.options().dtype(at::kInt));
-    // selected weights (w[argmax], w[argmin]) for the backward, only where the caller keeps them
-    at::Tensor w_sel;
-    if (want_w_sel) w_sel = at::empty({2, s.N, s.M}, a.options());
+    // selected operands for the backward, only where the caller keeps them: planes 0, 1 hold
+    // w[argmax], w[argmin], planes 2, 3 hold x[argmax], x[argmin]
+    at::Tensor sel;
+    if (with_sel) sel = at::empty({hand_over ? 4 : 0, s.N, s.M}, a.options());
+    float *w_sel = (with_sel && hand_over) ? sel.data_ptr<float>() : nullptr;
+    float *x_sel = w_sel ? w_sel + 2 * s.N * s.M : nullptr;
     if (s.N == 0 || s.M == 0) {
-        if (want_w_sel) return {c, argmax, argmin, w_sel};
+        if (with_sel) return {c, argmax, argmin, sel};
         return {c, argmax, argmin};
     }
     const size_t ws_bytes = mam_fc_forward_workspace(s.N, s.K, s.M);
@@ -116,10 +119,10 @@ std::vector<at::Tensor> forward_impl(const at::Tensor &a, const at::Tensor &w, i
     check_rc(mam_fc_forward(a.data_ptr<float>(), row_stride(a, "a"), w.data_ptr<float>(),
                             row_stride(w, "the weight operand"), layout, bias_ptr(bias),
                             c.data_ptr<float>(), argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
-                            want_w_sel ? w_sel.data_ptr<float>() : nullptr, s.N, s.K, s.M,
+                            w_sel, x_sel, s.N, s.K, s.M,
                             ws.defined() ? ws.data_ptr() : nullptr, ws_bytes, current_stream(a)),
              "mam_fc_forward");
-    if (want_w_sel) return {c, argmax, argmin, w_sel};
+    if (with_sel) return {c, argmax, argmin, sel};
     return {c, argmax, argmin};
 }
 
@@ -142,7 +145,7 @@ at::Tensor forward_values_impl(const at::Tensor &a, const at::Tensor &w, int lay
 
 std::vector<at::Tensor> backward_impl(const at::Tensor &a, const at::Tensor &w, int layout,
                                       const at::Tensor &grad, const at::Tensor &argmax,
-                                      const at::Tensor &argmin, const c10::optional<at::Tensor> &w_sel)
+                                      const at::Tensor &argmin, const c10::optional<at::Tensor> &sel)
 {
     const FwdShape s = check_forward(a, w, layout, c10::nullopt);
     check_f32_2d(grad, "grad");
@@ -150,13 +153,14 @@ std::vector<at::Tensor> backward_impl(const at::Tensor &a, const at::Tensor &w, 
     check_same_device(a, grad, "grad");
     check_index(argmax, grad, "argmax");
     check_index(argmin, grad, "argmin");
-    const float *w_sel_ptr = nullptr;
-    if (w_sel.has_value() && w_sel->defined()) {
-        TORCH_CHECK(w_sel->is_cuda() && w_sel->scalar_type() == at::kFloat && w_sel->is_contiguous() &&
-                        w_sel->dim() == 3 && w_sel->size(0) == 2 && w_sel->size(1) == s.N && w_sel->size(2) == s.M,
-                    "w_sel must be a contiguous float32 GPU tensor of shape (2, batch, out_features)");
-        check_same_device(a, *w_sel, "w_sel");
-        w_sel_ptr = w_sel->data_ptr<float>();
+    const float *w_sel_ptr = nullptr, *x_sel_ptr = nullptr;
+    if (sel.has_value() && sel->defined() && sel->numel() > 0) {
+        TORCH_CHECK(sel->is_cuda() && sel->scalar_type() == at::kFloat && sel->is_contiguous() &&
+                        sel->dim() == 3 && sel->size(0) == 4 && sel->size(1) == s.N && sel->size(2) == s.M,
+                    "sel must be a contiguous float32 GPU tensor of shape (4, batch, out_features)");
+        check_same_device(a, *sel, "sel");
+        w_sel_ptr = sel->data_ptr<float>();
+        x_sel_ptr = w_sel_ptr + 2 * s.N * s.M;
     }
     const c10::DeviceGuard guard(a.device());
     const at::Tensor g = grad.contiguous();
@@ -164,7 +168,7 @@ std::vector<at::Tensor> backward_impl(const at::Tensor &a, const at::Tensor &w, 
     auto w_grad = at::empty(w.sizes(), w.options());
     check_rc(mam_fc_backward(a.data_ptr<float>(), row_stride(a, "a"), w.data_ptr<float>(),
                              row_stride(w, "the weight operand"), layout, g.data_ptr<float>(),
-                             argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(), w_sel_ptr,
+                             argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(), w_sel_ptr, x_sel_ptr,
                              a_grad.data_ptr<float>(), w_grad.data_ptr<float>(), s.N, s.K, s.M,
                              current_stream(a)),
              "mam_fc_backward");
@@ -176,7 +180,7 @@ std::vector<at::Tensor> backward_impl(const at::Tensor &a, const at::Tensor &w, 
 // they were contiguous. ----
 std::vector<at::Tensor> fullyconnected(at::Tensor a, at::Tensor b)
 {
-    return forward_impl(a, b, MAM_W_KM, c10::nullopt, false);
+    return forward_impl(a, b, MAM_W_KM, c10::nullopt, false, false);
 }
 
 at::Tensor fullyconnected_fast(at::Tensor a, at::Tensor b)
@@ -192,9 +196,9 @@ std::vector<at::Tensor> fullyconnected_backward(at::Tensor a, at::Tensor b, at::
 
 // ---- additions: weight in the module's own (out_features, in_features) layout, fused bias ----
 std::vector<at::Tensor> fullyconnected_wt(const at::Tensor &a, const at::Tensor &weight,
-                                          const c10::optional<at::Tensor> &bias)
+                                          const c10::optional<at::Tensor> &bias, bool hand_over)
 {
-    return forward_impl(a, weight, MAM_W_MK, bias, true);
+    return forward_impl(a, weight, MAM_W_MK, bias, true, hand_over);
 }
 
 at::Tensor fullyconnected_fast_wt(const at::Tensor &a, const at::Tensor &weight,
@@ -206,9 +210,9 @@ at::Tensor fullyconnected_fast_wt(const at::Tensor &a, const at::Tensor &weight,
 std::vector<at::Tensor> fullyconnected_wt_backward(const at::Tensor &a, const at::Tensor &weight,
                                                    const at::Tensor &grad, const at::Tensor &argmax,
                                                    const at::Tensor &argmin,
-                                                   const c10::optional<at::Tensor> &w_sel)
+                                                   const c10::optional<at::Tensor> &sel)
 {
-    return backward_impl(a, weight, MAM_W_MK, grad, argmax, argmin, w_sel);
+    return backward_impl(a, weight, MAM_W_MK, grad, argmax, argmin, sel);
 }
 
 void selection_count(const at::Tensor &argmax, const at::Tensor &argmin, at::Tensor max_count,
@@ -389,9 +393,9 @@ TORCH_LIBRARY(mamtorch_kernel_v4, m)
     m.def("fullyconnected(Tensor a, Tensor b) -> Tensor[]");
     m.def("fullyconnected_fast(Tensor a, Tensor b) -> Tensor");
     m.def("fullyconnected_backward(Tensor a, Tensor b, Tensor grad, Tensor argmax, Tensor argmin) -> Tensor[]");
-    m.def("fullyconnected_wt(Tensor a, Tensor weight, Tensor? bias) -> Tensor[]");
+    m.def("fullyconnected_wt(Tensor a, Tensor weight, Tensor? bias, bool hand_over) -> Tensor[]");
     m.def("fullyconnected_fast_wt(Tensor a, Tensor weight, Tensor? bias) -> Tensor");
-    m.def("fullyconnected_wt_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin, Tensor? w_sel) -> Tensor[]");
+    m.def("fullyconnected_wt_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin, Tensor? sel) -> Tensor[]");
     m.def("selection_count(Tensor argmax, Tensor argmin, Tensor(a!) max_count, Tensor(b!) min_count, int mode) -> ()");
 }
 

@@ -6,9 +6,10 @@ served by the exact kernel, so its error against the oracle is zero.
 
 ``fullyconnected_wt`` is an addition: it takes the module's ``weight`` (out, in) as stored, so no
 transposed copy of the weight is made per call, adds the bias inside the kernel, and returns the
-weight gradient in (out, in) layout.  The raw operator returns a fourth tensor, the selected
-weights w[argmax] / w[argmin] of shape (2, N, out): the index resolution has them in hand, and
-the backward then needs no random reads of the weight matrix.
+weight gradient in (out, in) layout.  With ``hand_over`` the raw operator returns a fourth tensor of
+shape (4, N, out): the selected weights w[argmax], w[argmin] and the selected inputs x[argmax],
+x[argmin].  The index resolution has them in hand, and the backward then needs no random reads of
+the weight matrix or of the input.
 """
 import torch
 from torch import Tensor
@@ -27,14 +28,16 @@ def fullyconnected(a: Tensor, b: Tensor) -> list[Tensor]:
 
 def fullyconnected_wt(a: Tensor, weight: Tensor, bias=None) -> list[Tensor]:
     """a (N, in), weight (out, in), bias (out) or None -> [C, argmax, argmin]."""
-    return K.fullyconnected_wt.default(a, weight, bias)[:3]
+    # the selected operands are only worth writing when a backward will read them
+    hand_over = torch.is_grad_enabled() and (a.requires_grad or weight.requires_grad)
+    return K.fullyconnected_wt.default(a, weight, bias, hand_over)[:3]
 
 
 register_exact_forward(library_name)
 
 
 @torch.library.register_fake(f"{library_name}::fullyconnected_wt")
-def _(a, weight, bias):
+def _(a, weight, bias, hand_over):
     torch._check(a.dim() == 2 and weight.dim() == 2)
     torch._check(a.size(1) == weight.size(1))
     torch._check(a.dtype == torch.float)
@@ -44,11 +47,11 @@ def _(a, weight, bias):
     return [torch.empty(shape, dtype=torch.float, device=a.device),
             torch.empty(shape, dtype=torch.int, device=a.device),
             torch.empty(shape, dtype=torch.int, device=a.device),
-            torch.empty((2,) + shape, dtype=torch.float, device=a.device)]
+            torch.empty((4 if hand_over else 0,) + shape, dtype=torch.float, device=a.device)]
 
 
 @torch.library.register_fake(f"{library_name}::fullyconnected_wt_backward")
-def _(a, weight, grad, argmax, argmin, w_sel):
+def _(a, weight, grad, argmax, argmin, sel):
     torch._check(a.size(1) == weight.size(1))
     torch._check(grad.size(0) == a.size(0))
     torch._check(grad.size(1) == weight.size(0))
@@ -61,22 +64,22 @@ def _(a, weight, grad, argmax, argmin, w_sel):
 
 
 def _wt_setup_context(ctx, inputs, output):
-    a, weight, bias = inputs
-    _, argmax, argmin, w_sel = output
+    a, weight, bias = inputs[:3]
+    _, argmax, argmin, sel = output
     need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
     ctx.save_for_backward(a if need else None, weight if need else None, argmax, argmin,
-                          w_sel if need else None)
+                          sel if need else None)
 
 
 def _wt_backward(ctx, grad):
-    a, weight, argmax, argmin, w_sel = ctx.saved_tensors
+    a, weight, argmax, argmin, sel = ctx.saved_tensors
     a_grad, w_grad, bias_grad = None, None, None
     g = grad[0]
     if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-        a_grad, w_grad = K.fullyconnected_wt_backward.default(a, weight, g.contiguous(), argmax, argmin, w_sel)
+        a_grad, w_grad = K.fullyconnected_wt_backward.default(a, weight, g.contiguous(), argmax, argmin, sel)
     if ctx.needs_input_grad[2]:
         bias_grad = g.sum(dim=0)
-    return a_grad, w_grad, bias_grad
+    return a_grad, w_grad, bias_grad, None
 
 
 torch.library.register_autograd(

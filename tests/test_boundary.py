@@ -45,14 +45,14 @@ def test_workspace_queries_are_pure_host_calls():
 def test_argument_validation_without_a_gpu():
     l = capi.lib()
     # invalid arguments are rejected on the host before anything is launched
-    assert l.mam_fc_forward(None, 4, None, 4, 7, None, None, None, None, None, 2, 4, 2, None, 0, None) == -1
+    assert l.mam_fc_forward(None, 4, None, 4, 7, None, None, None, None, None, None, 2, 4, 2, None, 0, None) == -1
     assert b"w_layout" in l.mam_last_error()
-    assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, -1, 4, 2, None, 0, None) == -1
-    assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, 2, 4, 2, None, 0, None) == -1
+    assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, None, -1, 4, 2, None, 0, None) == -1
+    assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, None, 2, 4, 2, None, 0, None) == -1
     assert b"null" in l.mam_last_error()
     assert l.mam_selection_count(None, None, None, None, 2, 2, 2, 9, None) == -1
     # empty problems are a no-op
-    assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, 0, 4, 2, None, 0, None) == 0
+    assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, None, 0, 4, 2, None, 0, None) == 0
     assert l.mam_selection_count(None, None, None, None, 0, 2, 2, 0, None) == 0
 
 
@@ -105,12 +105,14 @@ def test_fake_kernels_propagate_shapes():
     assert torch.ops.mamtorch_kernel_v4.fullyconnected_fast(a, b).shape == (7, 5)
     c, amax, amin = torch.ops.mamtorch_kernel_v1.fullyconnected(a, b)
     assert c.shape == (7, 5)
-    c, amax, amin, w_sel = torch.ops.mamtorch_kernel_v4.fullyconnected_wt(a, w, None)
-    assert c.shape == (7, 5) and w_sel.shape == (2, 7, 5)
+    c, amax, amin, sel = torch.ops.mamtorch_kernel_v4.fullyconnected_wt(a, w, None, False)
+    assert sel.shape == (0, 7, 5)
+    c, amax, amin, sel = torch.ops.mamtorch_kernel_v4.fullyconnected_wt(a, w, None, True)
+    assert c.shape == (7, 5) and sel.shape == (4, 7, 5)
     g = torch.empty(7, 5, device="meta")
     ag, bg = torch.ops.mamtorch_kernel_v4.fullyconnected_backward(a, b, g, amax, amin)
     assert ag.shape == (7, 11) and bg.shape == (11, 5)
-    ag, wg = torch.ops.mamtorch_kernel_v4.fullyconnected_wt_backward(a, w, g, amax, amin, w_sel)
+    ag, wg = torch.ops.mamtorch_kernel_v4.fullyconnected_wt_backward(a, w, g, amax, amin, sel)
     assert ag.shape == (7, 11) and wg.shape == (5, 11)
     with pytest.raises(RuntimeError):
         torch.ops.mamtorch_kernel_v4.fullyconnected(a, torch.empty(12, 5, device="meta"))

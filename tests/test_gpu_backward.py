@@ -43,9 +43,17 @@ def _check(x, w_mk, grad, amax, amin, what, layouts=(0, 1)):
         # the same call with the selected weights handed over instead of gathered
         cols = torch.arange(w_mk.shape[0])[None, :]
         w_sel = torch.stack([w_mk[cols, torch.tensor(amax).long()], w_mk[cols, torch.tensor(amin).long()]]).to(dev)
+        rows = torch.arange(x.shape[0])[:, None]
+        x_sel = torch.stack([x[rows, torch.tensor(amax).long()], x[rows, torch.tensor(amin).long()]]).to(dev)
         xg2, _ = capi.fc_backward(xd, wd, gd, a1, a2, layout, want_w=False, w_sel=w_sel.contiguous())
+        xg3, wg3 = capi.fc_backward(xd, wd, gd, a1, a2, layout, w_sel=w_sel.contiguous(), x_sel=x_sel.contiguous())
+        _, wg4 = capi.fc_backward(xd, wd, gd, a1, a2, layout, want_x=False, x_sel=x_sel.contiguous())
         torch.cuda.synchronize()
         close(xg2.cpu().numpy(), xo, xs, "%s x_grad (w_sel) layout %d" % (what, layout))
+        close(xg3.cpu().numpy(), xo, xs, "%s x_grad (w_sel, x_sel) layout %d" % (what, layout))
+        for got, tag in ((wg3, "w_sel, x_sel"), (wg4, "x_sel")):
+            got = got.cpu().numpy() if layout == capi.W_MK else got.cpu().numpy().T
+            close(got, wo, ws_, "%s w_grad (%s) layout %d" % (what, tag, layout))
         wg = wg.cpu().numpy() if layout == capi.W_MK else wg.cpu().numpy().T
         close(xg.cpu().numpy(), xo, xs, "%s x_grad layout %d" % (what, layout))
         close(wg, wo, ws_, "%s w_grad layout %d" % (what, layout))

@@ -1,5 +1,6 @@
 """GPU parity of the dense MAM forward, driven through the C ABI (mamtorch_amd.capi).
 Bar: values bit-exact (fp32 bit patterns), argmax/argmin exactly equal, against the CPU oracle."""
+import contextlib
 import json
 import os
 
@@ -18,6 +19,17 @@ def _dev():
     return torch.device("cuda:0")
 
 
+@contextlib.contextmanager
+def forward_tiling(name):
+    """MAM_FORWARD_TILING (read by the library at every call) for the calls inside the block."""
+    if name:
+        os.environ["MAM_FORWARD_TILING"] = name
+    try:
+        yield
+    finally:
+        os.environ.pop("MAM_FORWARD_TILING", None)
+
+
 def _run_both_layouts(x, w_mk, bias=None, what=""):
     """x (N,K), w_mk (M,K) CPU tensors.  Checks forward (+values-only) in both layouts vs the oracle."""
     from mamtorch_amd import capi
@@ -31,14 +43,10 @@ def _run_both_layouts(x, w_mk, bias=None, what=""):
     for layout, w, tiling in ((capi.W_MK, w_mk.contiguous(), None), (capi.W_MK, w_mk.contiguous(), "wide"),
                               (capi.W_KM, w_mk.T.contiguous(), None)):
         wd = w.to(dev)
-        if tiling:
-            os.environ["MAM_FORWARD_TILING"] = tiling
-        try:
+        with forward_tiling(tiling):
             c, amax, amin = capi.fc_forward(xd, wd, layout, bd)
             cv = capi.fc_forward_values(xd, wd, layout, bd)
             torch.cuda.synchronize()
-        finally:
-            os.environ.pop("MAM_FORWARD_TILING", None)
         tag = "%s layout=%d tiling=%s" % (what, layout, tiling or "default")
         assert_bits_equal(c.cpu().numpy(), want[0], tag + " c")
         assert_index_equal(amax.cpu().numpy(), want[1], tag + " argmax")
@@ -310,7 +318,8 @@ def test_large_batch_inference_config4(M):
 
 @pytest.mark.parametrize("shape", [(64, 784, 256), (256, 4096, 512), (70, 123, 45), (300, 2048, 200)])
 def test_selected_weights_output(shape):
-    """w_sel[0] = w[argmax[n,m], m], w_sel[1] = w[argmin[n,m], m] (exact copies), both layouts."""
+    """w_sel[0] = w[argmax[n,m], m], w_sel[1] = w[argmin[n,m], m], x_sel[0] = x[n, argmax[n,m]],
+    x_sel[1] = x[n, argmin[n,m]] (exact copies), both layouts, both tilings."""
     from mamtorch_amd import capi
 
     dev = _dev()
@@ -318,10 +327,24 @@ def test_selected_weights_output(shape):
     x, w, _ = random_case(N, K, M, seed=11)
     want = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
     cols = np.arange(M)[None, :]
-    for layout, wl in ((capi.W_MK, w.contiguous()), (capi.W_KM, w.T.contiguous())):
+    rows = np.arange(N)[:, None]
+    for layout, wl, tiling in ((capi.W_MK, w.contiguous(), None), (capi.W_MK, w.contiguous(), "wide"),
+                               (capi.W_KM, w.T.contiguous(), None)):
         w_sel = torch.full((2, N, M), float("nan"), device=dev)
-        c, amax, amin = capi.fc_forward(x.to(dev), wl.to(dev), layout, w_sel=w_sel)
-        torch.cuda.synchronize()
-        assert_index_equal(amax.cpu().numpy(), want[1], "argmax")
-        assert_bits_equal(w_sel[0].cpu().numpy(), w.numpy()[cols, want[1]], "w_sel max layout %d" % layout)
-        assert_bits_equal(w_sel[1].cpu().numpy(), w.numpy()[cols, want[2]], "w_sel min layout %d" % layout)
+        x_sel = torch.full((2, N, M), float("nan"), device=dev)
+        with forward_tiling(tiling):
+            c, amax, amin = capi.fc_forward(x.to(dev), wl.to(dev), layout, w_sel=w_sel, x_sel=x_sel)
+            torch.cuda.synchronize()
+        what = "layout %d tiling %s" % (layout, tiling)
+        assert_bits_equal(c.cpu().numpy(), want[0], "c " + what)
+        assert_index_equal(amax.cpu().numpy(), want[1], "argmax " + what)
+        assert_bits_equal(w_sel[0].cpu().numpy(), w.numpy()[cols, want[1]], "w_sel max " + what)
+        assert_bits_equal(w_sel[1].cpu().numpy(), w.numpy()[cols, want[2]], "w_sel min " + what)
+        assert_bits_equal(x_sel[0].cpu().numpy(), x.numpy()[rows, want[1]], "x_sel max " + what)
+        assert_bits_equal(x_sel[1].cpu().numpy(), x.numpy()[rows, want[2]], "x_sel min " + what)
+        # only one of the two asked for
+        x_only = torch.full((2, N, M), float("nan"), device=dev)
+        with forward_tiling(tiling):
+            capi.fc_forward(x.to(dev), wl.to(dev), layout, x_sel=x_only)
+            torch.cuda.synchronize()
+        assert torch.equal(x_only, x_sel)

@@ -62,7 +62,7 @@ def test_opcheck():
     torch.library.opcheck(torch.ops.mamtorch_kernel_v1.fullyconnected, (a, b), test_utils=tests)
     torch.library.opcheck(torch.ops.mamtorch_kernel_v4.fullyconnected, (a, b), test_utils=tests)
     torch.library.opcheck(torch.ops.mamtorch_kernel_v4.fullyconnected_fast, (a, b), test_utils=tests)
-    torch.library.opcheck(torch.ops.mamtorch_kernel_v4.fullyconnected_wt, (a, wt, bias), test_utils=tests)
+    torch.library.opcheck(torch.ops.mamtorch_kernel_v4.fullyconnected_wt, (a, wt, bias, True), test_utils=tests)
     torch.library.opcheck(torch.ops.mamtorch_kernel_v4.fullyconnected_fast_wt, (a, wt, None), test_utils=tests)
     _, amax, amin = torch.ops.mamtorch_kernel_v4.fullyconnected(a.detach(), b.detach())
     torch.library.opcheck(torch.ops.mamtorch_kernel_v4.fullyconnected_backward,
