@@ -557,9 +557,11 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
         int *grps = reinterpret_cast<int *>(tile_b) + wave * (TJ * 2 * 64);
         static_assert((NT / 64) * (TJ * 2 * 64 + RES_WORDS) <= TILE_FLOATS, "resolve scratch does not fit");
         float *res = tile_a + (NT / 64) * (TJ * 2 * 64) + wave * RES_WORDS;
+        // From here on a wave touches only its own corner of LDS, and the LDS operations of one wave
+        // complete in issue order: no workgroup barrier between parking and resolving.
+        __syncthreads();
 #pragma unroll
         for (int i = 0; i < TI; ++i) {
-            __syncthreads();
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
                 vals[(j * 2 + 0) * 64 + lane] = vmax[i][j];
@@ -567,7 +569,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
                 grps[(j * 2 + 0) * 64 + lane] = g0 + gmax[i][j];
                 grps[(j * 2 + 1) * 64 + lane] = g0 + gmin[i][j];
             }
-            __syncthreads();
+            __builtin_amdgcn_wave_barrier();
 #pragma unroll 1
             for (int j = 0; j < TJ; ++j) {
                 const int nbase = row0 + 16 * i + 4 * wave, mbase = col0 + 16 * j;
@@ -885,9 +887,11 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
         int *grps = reinterpret_cast<int *>(tile_b) + wave * (sx::TJ * 128);
         static_assert((sx::NT / 64) * (sx::TJ * 128 + RES_WORDS) <= sx::TILE_FLOATS, "resolve scratch does not fit");
         float *res = tile_a + (sx::NT / 64) * (sx::TJ * 128) + wave * RES_WORDS;
+        // From here on a wave touches only its own corner of LDS, and the LDS operations of one wave
+        // complete in issue order: no workgroup barrier between parking and resolving.
+        __syncthreads();
 #pragma unroll
         for (int i = 0; i < sx::TI; ++i) {
-            __syncthreads();
 #pragma unroll
             for (int j = 0; j < sx::TJ; ++j) {
                 vals[(j * 2 + 0) * 64 + lane] = vmax[i][j];
@@ -895,7 +899,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
                 grps[(j * 2 + 0) * 64 + lane] = g0 + gmax[i][j];
                 grps[(j * 2 + 1) * 64 + lane] = g0 + gmin[i][j];
             }
-            __syncthreads();
+            __builtin_amdgcn_wave_barrier();
             const int nrow = row0 + i;
 #pragma unroll 1
             for (int j = 0; j < sx::TJ; ++j) {
