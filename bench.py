@@ -75,11 +75,16 @@ class Layer:
         query = lib.mam_fc_forward_values_workspace if values_only else lib.mam_fc_forward_workspace
         self.ws_bytes = query(N, K, M)
         self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
-        self.sp = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+        self.torch, self.dev = torch, dev
 
     @staticmethod
     def _p(t):
         return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+    @property
+    def sp(self):
+        # the stream that is current at the call (the capture stream while a graph is recorded)
+        return ctypes.c_void_p(self.torch.cuda.current_stream(self.dev).cuda_stream)
 
     def forward(self):
         P, N, K, M = self._p, self.N, self.K, self.M
@@ -139,12 +144,28 @@ def dense_cpu_baseline(torch, layers_cpu, budget_s, with_backward):
     }
 
 
-def time_phases(torch, stream, phases, steps, warmup):
-    """Runs every phase once per step; returns (ms per step by the host clock, ms per phase by events)."""
+def time_phases(torch, stream, phases, steps, warmup, graph=False):
+    """Runs every phase once per step; returns (ms per step by the host clock, ms per phase by events).
+    graph: the step is recorded once into a HIP graph and the timed steps are replays of it; the
+    per-phase times then come from a second, eager pass."""
     for _ in range(warmup):
         for _, fn in phases:
             fn()
     torch.cuda.synchronize()
+    ms_graph = None
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _, fn in phases:
+                fn()
+        for _ in range(min(warmup, 20)):
+            g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.replay()
+        torch.cuda.synchronize()
+        ms_graph = (time.perf_counter() - t0) * 1e3 / steps
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(len(phases) + 1)] for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -159,7 +180,7 @@ def time_phases(torch, stream, phases, steps, warmup):
     for i, (label, _) in enumerate(phases):
         ms = sum(e[i].elapsed_time(e[i + 1]) for e in ev) / steps
         per_phase[label] = per_phase.get(label, 0.0) + ms
-    return (t1 - t0) * 1e3 / steps, per_phase
+    return (ms_graph if graph else (t1 - t0) * 1e3 / steps), per_phase
 
 
 def valu_roofline(kernel, triples, ms):
@@ -225,11 +246,12 @@ def run_dense(torch, capi, lib, dev, args):
         del calibration_copy
 
     stream = torch.cuda.current_stream(dev)
-    ms_step, ph = time_phases(torch, stream, phases, args.steps, args.warmup)
+    ms_step, ph = time_phases(torch, stream, phases, args.steps, args.warmup, args.graph)
     triples = sum(L.N * L.K * L.M for L in layers)
     fwd_ms = ph["forward"]
     out = {
-        "config": {"workload": text, "name": wl, "layers": [{"N": L.N, "K": L.K, "M": L.M} for L in layers]},
+        "config": {"workload": text, "name": wl, "layers": [{"N": L.N, "K": L.K, "M": L.M} for L in layers],
+                   "launch": "one HIP graph replay per step" if args.graph else "one C-ABI call per phase"},
         "phases_ms": {k: round(v, 5) for k, v in ph.items()},
         "forward_gops": round(triples / (fwd_ms * 1e-3) / 1e9, 2),
     }
@@ -424,6 +446,8 @@ def main():
                     help="untimed steps; the GPU clock needs ~100 launches to ramp up")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--workload", choices=WORKLOADS, default="headline")
+    ap.add_argument("--graph", action="store_true",
+                    help="dense workloads: record one step into a HIP graph and time replays of it")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the MAM hot path has no multi-GPU part in this build "
