@@ -20,7 +20,14 @@ namespace mam {
 namespace selcount {
 
 
-constexpr int NT_H = 512;
+#ifndef MAM_SELCOUNT_NT
+#define MAM_SELCOUNT_NT 512
+#endif
+constexpr int NT_H = MAM_SELCOUNT_NT;
+#ifndef MAM_SELCOUNT_FU
+#define MAM_SELCOUNT_FU 2
+#endif
+constexpr int FU = MAM_SELCOUNT_FU;   // 16-byte chunks a thread has in flight while the slab is streamed back
 
 template <int MODE>
 __device__ __forceinline__ void mark(uint32_t *word, uint32_t field)
@@ -83,12 +90,12 @@ __global__ __launch_bounds__(NT_H) void count_kernel(const int32_t *__restrict__
         if (vec) {
             const int q = kn >> 2;
             const int total = rn * q;
-            for (int eb = tid; eb < total; eb += 4 * NT_H) {
-                uint4 v[4];
-                int4 amx[4], amn[4];
-                int64_t cell[4];
+            for (int eb = tid; eb < total; eb += FU * NT_H) {
+                uint4 v[FU];
+                int4 amx[FU], amn[FU];
+                int64_t cell[FU];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < FU; ++u) {
                     const int e = eb + u * NT_H;
                     v[u] = make_uint4(0u, 0u, 0u, 0u);
                     cell[u] = 0;
@@ -101,7 +108,7 @@ __global__ __launch_bounds__(NT_H) void count_kernel(const int32_t *__restrict__
                 if (MODE == MAM_COUNT_REFERENCE) {
                     // both flags land in max_count: fold them into the low field
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < FU; ++u) {
                         v[u].x = (v[u].x & 1u) + (v[u].x >> 16);
                         v[u].y = (v[u].y & 1u) + (v[u].y >> 16);
                         v[u].z = (v[u].z & 1u) + (v[u].z >> 16);
@@ -109,13 +116,13 @@ __global__ __launch_bounds__(NT_H) void count_kernel(const int32_t *__restrict__
                     }
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < FU; ++u) {
                     const uint32_t any = v[u].x | v[u].y | v[u].z | v[u].w;
                     if (any & 0xffffu) amx[u] = *reinterpret_cast<const int4 *>(max_count + cell[u]);
                     if (any >> 16) amn[u] = *reinterpret_cast<const int4 *>(min_count + cell[u]);
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < FU; ++u) {
                     const uint32_t any = v[u].x | v[u].y | v[u].z | v[u].w;
                     if (any & 0xffffu) {
                         amx[u].x += (int)(v[u].x & 0xffffu); amx[u].y += (int)(v[u].y & 0xffffu);
