@@ -189,9 +189,12 @@ __device__ __forceinline__ int quad_min(int v)
     return o < v ? o : v;
 }
 
-template <class NM>
+//   operands(r, slot, sub, kb, xp, wp): where the 4 x and 4 w operands k = kb .. kb+3 of the task in round r
+//   live.  The addresses are most of the instructions of a round when they are formed in 64 bits per
+//   lane, so a caller whose 64 outputs share bases hands in something cheaper.
+template <class NM, class OP>
 __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps, float *res,
-                                             int lane, NM nm_of)
+                                             int lane, NM nm_of, OP operands)
 {
     float *res_v = res;                                    // [2][64]
     int *res_i = reinterpret_cast<int *>(res + 128);        // [2][64]
@@ -205,14 +208,12 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
     for (int r = 0; r < RES_ROUNDS; ++r) {
         const int task = r * TPR + lane / LPT;
         const int slot = task >> 1, ext = task & 1, sub = lane % LPT;
-        int n, m;
-        bool valid;
-        nm_of(slot, n, m, valid);
         target[r] = vals[ext * 64 + slot];
         grp[r] = grps[ext * 64 + slot];
-        const int kb = grp[r] * G + sub * 4;
-        xa[r] = *reinterpret_cast<const float4 *>(p.x + (int64_t)n * p.ldx + kb);
-        wa[r] = *reinterpret_cast<const float4 *>(p.w + (int64_t)m * p.ldw + kb);
+        const float *xp, *wp;
+        operands(r, slot, sub, grp[r] * G + sub * 4, xp, wp);
+        xa[r] = *reinterpret_cast<const float4 *>(xp);
+        wa[r] = *reinterpret_cast<const float4 *>(wp);
     }
 #pragma unroll
     for (int r = 0; r < RES_ROUNDS; ++r) {
@@ -257,6 +258,21 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
             p.xsel[(int64_t)p.N * p.M + o] = res_x[64 + lane];
         }
     }
+}
+
+// The general case: every output has its own row of x and of w.
+template <class NM>
+__device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps, float *res,
+                                             int lane, NM nm_of)
+{
+    resolve_wave(p, vals, grps, res, lane, nm_of,
+                 [&](int, int slot, int, int kb, const float *&xp, const float *&wp) {
+                     int n, m;
+                     bool valid;
+                     nm_of(slot, n, m, valid);
+                     xp = p.x + (int64_t)n * p.ldx + kb;
+                     wp = p.w + (int64_t)m * p.ldw + kb;
+                 });
 }
 
 // Stages one k-tile [k0, k0+KT) of X and W into LDS for any alignment and any ragged edge:
@@ -682,6 +698,14 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
         grps_s[wave][1][lane] = gmin;
         __syncthreads();
         const int nbase = pn * 16 + 4 * wave, mbase = pm * 16;
+        // slot = 8 r + lane / 8 in round r: batch row nbase + r / 2 (the same for the whole wave) and
+        // neuron mbase + 8 (r & 1) + lane / 8, so the operands sit at 32-bit byte offsets from
+        // wave-uniform bases (the host checked that 16 rows of w span < 4 GiB)
+        const int mb = mbase < p.M ? mbase : p.M - 1;
+        const char *wrows = reinterpret_cast<const char *>(p.w + (int64_t)mb * p.ldw);
+        const uint32_t ldw4 = (uint32_t)p.ldw * 4u;
+        const uint32_t last = (uint32_t)(p.M - 1 - mb) * ldw4;
+        const uint32_t mine = (uint32_t)(lane >> 3) * ldw4;
         resolve_wave(p, &vals_s[wave][0][0], &grps_s[wave][0][0], &res_s[wave][0], lane,
                      [&](int slot, int &n, int &m, bool &valid) {
                          n = nbase + (slot >> 4);
@@ -689,6 +713,14 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
                          valid = n < p.N && m < p.M;
                          n = n < p.N ? n : p.N - 1;
                          m = m < p.M ? m : p.M - 1;
+                     },
+                     [&](int r, int, int, int kb, const float *&xp, const float *&wp) {
+                         const int n = (nbase + (r >> 1)) < p.N ? (nbase + (r >> 1)) : (p.N - 1);
+                         const char *xrow = reinterpret_cast<const char *>(p.x + (int64_t)n * p.ldx);
+                         const uint32_t row = mine + (uint32_t)(8 * (r & 1)) * ldw4;
+                         const uint32_t k4 = (uint32_t)kb * 4u;
+                         xp = reinterpret_cast<const float *>(xrow + k4);
+                         wp = reinterpret_cast<const float *>(wrows + ((row < last ? row : last) + k4));
                      });
     } else if (live) {
         finish<LAYOUT, ARGS>(p, n_own, m_own, vmax, vmin, gmax, gmin);
@@ -901,9 +933,17 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
             }
             __builtin_amdgcn_wave_barrier();
             const int nrow = row0 + i;
+            // the 64 outputs of a set share the x row, and their w rows are mbase + slot: 32-bit byte
+            // offsets from two wave-uniform bases (the host checked that a tile of w spans < 4 GiB)
+            const char *xrow = reinterpret_cast<const char *>(p.x + (int64_t)(nrow < p.N ? nrow : p.N - 1) * p.ldx);
+            const uint32_t ldw4 = (uint32_t)p.ldw * 4u;
 #pragma unroll 1
             for (int j = 0; j < sx::TJ; ++j) {
                 const int mbase = col0 + 64 * j;
+                const int mb = mbase < p.M ? mbase : p.M - 1;
+                const char *wrows = reinterpret_cast<const char *>(p.w + (int64_t)mb * p.ldw);
+                const uint32_t last = (uint32_t)(p.M - 1 - mb) * ldw4;     // neurons past M repeat the last one
+                const uint32_t mine = (uint32_t)(lane >> 3) * ldw4;         // slot = 8 r + lane / 8
                 resolve_wave(p, vals + j * 128, grps + j * 128, res, lane,
                              [&](int slot, int &n, int &m, bool &valid) {
                                  n = nrow;
@@ -911,6 +951,12 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
                                  valid = n < p.N && m < p.M;
                                  n = n < p.N ? n : p.N - 1;
                                  m = m < p.M ? m : p.M - 1;
+                             },
+                             [&](int r, int, int, int kb, const float *&xp, const float *&wp) {
+                                 const uint32_t row = mine + (uint32_t)(8 * r) * ldw4;
+                                 const uint32_t k4 = (uint32_t)kb * 4u;
+                                 xp = reinterpret_cast<const float *>(xrow + k4);
+                                 wp = reinterpret_cast<const float *>(wrows + ((row < last ? row : last) + k4));
                              });
             }
         }
@@ -1022,7 +1068,8 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     // the fast staging path addresses a tile with 32-bit element offsets from the tile base
     const int64_t w_rows = (w_layout == MAM_W_MK) ? fwd::BM : fwd::KT;
     p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30));
-    p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0);
+    // (16 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
+    p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 25));
     // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
     if ((int64_t)p.k_per_split / G > 65536)
         return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds %d per K range", (long long)K, 65536 * G);
