@@ -137,9 +137,25 @@ __device__ __forceinline__ void gather_quad(const float *xr, const int4 &i1, con
 template <int LAYOUT>
 __device__ __forceinline__ void store_slab(const float *hist, float *__restrict__ w_grad, int tid, int m0,
                                            int k0, int rn, int kn, int kc, int log2r, int K, int M,
-                                           int vec_out)
+                                           int vec_out, bool accumulate)
 {
     const int R = 1 << log2r;
+    if (accumulate) {
+        // the batch is split over several workgroups per slab: w_grad was cleared beforehand and
+        // every workgroup adds its share (cells it never touched are skipped)
+        for (int e = tid; e < (LAYOUT == MAM_W_MK ? rn * kn : (kn << log2r)); e += NT_W) {
+            int r, kk;
+            float v;
+            if (LAYOUT == MAM_W_MK) { r = e / kn; kk = e - r * kn; v = hist[r * kc + kk]; }
+            else { kk = e >> log2r; r = e & (R - 1); v = hist[e]; }
+            if (v != 0.0f && r < rn) {
+                float *cell = LAYOUT == MAM_W_MK ? w_grad + (int64_t)(m0 + r) * K + k0 + kk
+                                                 : w_grad + (int64_t)(k0 + kk) * M + m0 + r;
+                __hip_atomic_fetch_add(cell, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        return;
+    }
     if (LAYOUT == MAM_W_MK) {
         if (vec_out) {  // K, k0 and kc are multiples of 4 and w_grad is 16-byte aligned
             const int q = kn >> 2;
@@ -173,19 +189,23 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
     const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
-    int kc, int vec_out, int mtiles, int tiles_per_wg)
+    int kc, int vec_out, int mtiles, int tiles_per_wg, int rows_per_split)
 {
     extern __shared__ float hist[];
     const int tid = threadIdx.x;
     const int R = 1 << log2r;
     const int qpr = R >> 2;
-    const int64_t items = (int64_t)N * qpr;
+    // blockIdx.z: which share of the batch rows (one share = the whole batch unless the host split it)
+    const int n_begin = blockIdx.z * rows_per_split;
+    const int n_rows = (N - n_begin) < rows_per_split ? (N - n_begin) : rows_per_split;
+    const bool accumulate = gridDim.z > 1;
+    const int64_t items = (int64_t)n_rows * qpr;
     const int k0 = blockIdx.y * kc;
     const int kn = (K - k0) < kc ? (K - k0) : kc;
     const int first = xcd_remap(blockIdx.x, gridDim.x) * tiles_per_wg;
 
     // this thread's first item of a slab: row n_first, neurons m0 + r_first .. +3
-    const int n_first = tid / qpr, r_first = (tid - n_first * qpr) * 4;
+    const int n_first = n_begin + tid / qpr, r_first = (tid % qpr) * 4;
     float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
     float4 s1 = g, s2 = g;      // selected inputs handed over by the forward, if any
     int4 i1 = make_int4(-1, -1, -1, -1), i2 = make_int4(-1, -1, -1, -1);
@@ -217,7 +237,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
         __syncthreads();
         if (have) scatter_quad<LAYOUT>(hist, g, i1, i2, x1, x2, r_first, k0, kn, kc, log2r);
         for (int64_t it = tid + NT_W; it < items; it += NT_W) {
-            const int n = (int)(it / qpr), r0 = (int)(it - (int64_t)n * qpr) * 4;
+            const int n = n_begin + (int)(it / qpr), r0 = (int)(it % qpr) * 4;
             if (m0 + r0 >= M) continue;
             const int64_t o = (int64_t)n * M + m0 + r0;
             const float4 gg = *reinterpret_cast<const float4 *>(grad + o);
@@ -236,7 +256,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
         }
         __syncthreads();
         if (t + 1 < tiles_per_wg && mt + 1 < mtiles) load_first(m0 + R);
-        store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out);
+        store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, accumulate);
         __syncthreads();
     }
 }
@@ -277,7 +297,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
                            (x_sel ? x_sel[nm + o] : xr[a2]) * g);
     }
     __syncthreads();
-    store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out);
+    store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, false);
 }
 
 // LDS a workgroup may use for a histogram, in floats.  gfx950 has 160 KiB per CU; above
@@ -311,7 +331,16 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         // 1024 k in 128 KiB.
         static const int big = lds_budget_floats((const void *)mam_bwd_w_kernel<LAYOUT>);
         static const int big2 = lds_budget_floats((const void *)mam_bwd_w_vec_kernel<LAYOUT>);
-        const int log2r = LAYOUT == MAM_W_MK ? 2 : 5;
+        const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
+                           ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)x_sel % 16 == 0) && (N * M % 4 == 0);
+        int log2r = LAYOUT == MAM_W_MK ? 2 : 5;
+        // Large batches: a thread reads 16 bytes of a batch row per array, so a slab of 4 neurons uses
+        // a quarter of every 64-byte sector it touches.  When K is small enough, 16 neurons (whole
+        // sectors) share a slab, and the batch is split over several workgroups per slab to keep the
+        // chip filled; they add their shares to the cleared w_grad.
+        const bool large_batch = LAYOUT == MAM_W_MK && vec_in && N >= 2048;
+        if (large_batch)
+            while (log2r < 4 && ((int64_t)2 << log2r) * ((K + 3) / 4 * 4) * 4 <= 64 * 1024) ++log2r;
         const int R = 1 << log2r;
         const int lds_cap = big < big2 ? big : big2;
         const int budget = LAYOUT == MAM_W_MK ? (R * 4096 < lds_cap ? R * 4096 : lds_cap) : lds_cap;
@@ -320,17 +349,34 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         const int64_t mtiles = ceil_div(M, R), ktiles = ceil_div(K, kc);
         if (ktiles > 65535) return fail(MAM_ERR_UNSUPPORTED, "K too large for the w_grad grid");
         const int vec_out = (K % 4 == 0) && ((uintptr_t)w_grad % 16 == 0);
-        const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
-                           ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)x_sel % 16 == 0) && (N * M % 4 == 0);
         if (vec_in) {
             // slabs per workgroup: enough workgroups for two per CU, the rest goes into pipelining
             int tpw = (int)(mtiles * ktiles / (2 * kNumCU));
             if (tpw < 1) tpw = 1;
             if (tpw > 8) tpw = 8;
+            // shares of the batch per slab: two rounds of as many workgroups as fit the chip (LDS, threads)
+            int64_t shares = 1;
+            if (large_batch) {
+                int64_t per_cu = (160 * 1024) / ((int64_t)R * kc * 4);
+                if (per_cu > 2048 / NT_W) per_cu = 2048 / NT_W;
+                if (per_cu < 1) per_cu = 1;
+                shares = (2 * per_cu * kNumCU + mtiles * ktiles / 2) / (mtiles * ktiles);
+                // a share adds a whole slab to w_grad with atomics: worth it only against >= K rows of work
+                if (shares > N / (K > 512 ? K : 512)) shares = N / (K > 512 ? K : 512);
+                if (shares > 65535) shares = 65535;
+                if (shares < 1) shares = 1;
+            }
+            const int64_t rows_per_share = ceil_div(N, shares);
+            shares = ceil_div(N, rows_per_share);
+            if (shares > 1) {
+                rc = fill_zero(w_grad, M * K, st);
+                if (rc != MAM_OK) return rc;
+            }
             hipLaunchKernelGGL((mam_bwd_w_vec_kernel<LAYOUT>),
-                               dim3((unsigned)ceil_div(mtiles, tpw), (unsigned)ktiles), dim3(NT_W),
+                               dim3((unsigned)ceil_div(mtiles, tpw), (unsigned)ktiles, (unsigned)shares), dim3(NT_W),
                                (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax, argmin, x_sel, N * M,
-                               w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out, (int)mtiles, tpw);
+                               w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out, (int)mtiles, tpw,
+                               (int)rows_per_share);
         } else {
             hipLaunchKernelGGL((mam_bwd_w_kernel<LAYOUT>), dim3((unsigned)mtiles, (unsigned)ktiles),
                                dim3(NT_W), (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax,

@@ -182,3 +182,18 @@ def test_vit_mlp_config3_shapes(dims):
     grad = torch.randn(N, M, generator=g)
     _, amax, amin = capi.fc_forward(x.to(dev), w.to(dev), capi.W_MK)
     _check(x, w, grad, amax.cpu().numpy(), amin.cpu().numpy(), "config 3", layouts=(1,))
+
+
+@pytest.mark.parametrize("shape", [(2100, 100, 36), (2048, 64, 4), (4099, 517, 132), (2500, 16, 20)])
+def test_large_batch_shares_of_the_batch_add_up(shape):
+    """From 2048 batch rows on, slabs of the (out, in) weight gradient may be wider than 4 neurons and the
+    batch is split over several workgroups per slab that add their shares: ragged last slab, ragged
+    last share, and selections piled up on a few k."""
+    N, K, M = shape
+    g = torch.Generator().manual_seed(N + K)
+    x = torch.randn(N, K, generator=g)
+    w = torch.randn(M, K, generator=g)
+    grad = torch.randn(N, M, generator=g)
+    amax = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32)
+    amin = torch.randint(0, min(K, 3), (N, M), generator=g, dtype=torch.int32)
+    _check(x, w, grad, amax.numpy(), amin.numpy(), "large batch %s" % (shape,))
