@@ -102,6 +102,78 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
     }
 }
 
+// x_grad for large batches: a workgroup owns R = 4 .. 16 batch rows with their whole K cells in LDS,
+// and the lanes of a wave are spread over those rows (64 / R lanes per row, 4 consecutive neurons
+// each).  The selections of ONE batch row pile up on the few k where |x| is largest, so in
+// mam_bwd_x_kernel most lanes of an instruction meet a contender; here only the 64 / R lanes of the
+// same row can, a compare-and-swap round settles nearly all of them, and the loads of a wave are
+// whole 64-byte (R = 16) to 256-byte (R = 4) pieces of R rows.
+template <int LAYOUT>
+__global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
+    const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
+    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
+    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int N, int K, int M, int log2r)
+{
+    extern __shared__ float hist[];   // [R][K]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int R = 1 << log2r;
+    const int lpr = 64 >> log2r;                  // lanes per batch row
+    const int r = lane / lpr, j = lane - r * lpr;
+    const int n = blockIdx.x * R + r;
+    const bool row_ok = n < N;
+    const int m_step = (NT_W / 64) * lpr * 4;     // neurons of a row the workgroup covers per trip
+    for (int i = tid; i < R * K; i += NT_W) hist[i] = 0.0f;
+    __syncthreads();
+
+    float4 g = make_float4(0.f, 0.f, 0.f, 0.f), s1 = g, s2 = g;
+    int4 i1, i2;
+    auto load = [&](int m) {
+        if (row_ok && m < M) {
+            const int64_t o = (int64_t)n * M + m;
+            g = *reinterpret_cast<const float4 *>(grad + o);
+            i1 = *reinterpret_cast<const int4 *>(argmax + o);
+            i2 = *reinterpret_cast<const int4 *>(argmin + o);
+            if (w_sel) {
+                s1 = *reinterpret_cast<const float4 *>(w_sel + o);
+                s2 = *reinterpret_cast<const float4 *>(w_sel + nm + o);
+            }
+        } else {
+            i1 = make_int4(-1, -1, -1, -1);
+            i2 = i1;
+        }
+    };
+    int m = (wave * lpr + j) * 4;
+    load(m);
+    float *row = hist + r * K;
+    const int trips = (M + m_step - 1) / m_step;     // the same for every thread: lanes past M hold no item
+    for (int t = 0; t < trips; ++t) {
+        const float4 cg = g, c1 = s1, c2 = s2;
+        const int4 a1 = i1, a2 = i2;
+        const int mc = m;
+        m += m_step;
+        load(m);         // the next trip's loads are in flight while this one is scattered
+        const float gv[4] = {cg.x, cg.y, cg.z, cg.w};
+        const int k1[4] = {a1.x, a1.y, a1.z, a1.w}, k2[4] = {a2.x, a2.y, a2.z, a2.w};
+        float w1[4] = {c1.x, c1.y, c1.z, c1.w}, w2[4] = {c2.x, c2.y, c2.z, c2.w};
+        if (!w_sel) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                w1[u] = (unsigned)k1[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k1[u], mc + u) : 0.0f;
+                w2[u] = (unsigned)k2[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k2[u], mc + u) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if ((unsigned)k1[u] < (unsigned)K) lds_add_sparse(&row[k1[u]], w1[u] * gv[u]);
+            if ((unsigned)k2[u] < (unsigned)K) lds_add_sparse(&row[k2[u]], w2[u] * gv[u]);
+        }
+    }
+    __syncthreads();
+    const int rows = (N - blockIdx.x * R) < R ? (N - blockIdx.x * R) : R;
+    float *dst = x_grad + (int64_t)blockIdx.x * R * K;
+    for (int i = tid; i < rows * K; i += NT_W) dst[i] = hist[i];
+}
+
 // Scatter of one (batch row, 4 consecutive neurons) item into the slab histogram.
 template <int LAYOUT>
 __device__ __forceinline__ void scatter_quad(float *hist, const float4 &g, const int4 &i1, const int4 &i2,
@@ -317,7 +389,22 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
                          float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
 {
     int rc = MAM_OK;
-    if (x_grad) {
+    const bool x_rows = N >= 2048 && K * 16 <= 64 * 1024 && (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
+                        ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) &&
+                        ((uintptr_t)w_sel % 16 == 0);
+    if (x_grad && x_rows) {
+        // as many rows per workgroup (4, 8 or 16) as fit 64 KiB of LDS
+        int log2r = 2;
+        while (log2r < 4 && ((int64_t)2 << log2r) * K * 4 <= 64 * 1024) ++log2r;
+        const int R = 1 << log2r;
+        static const int ok = lds_budget_floats((const void *)mam_bwd_x_rows_kernel<LAYOUT>);
+        (void)ok;
+        hipLaunchKernelGGL((mam_bwd_x_rows_kernel<LAYOUT>), dim3((unsigned)ceil_div(N, R)), dim3(NT_W),
+                           (size_t)R * K * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M, x_grad,
+                           (int)N, (int)K, (int)M, log2r);
+        rc = check_launch("mam_bwd_x_rows_kernel");
+        if (rc != MAM_OK) return rc;
+    } else if (x_grad) {
         static const int budget = lds_budget_floats((const void *)mam_bwd_x_kernel<LAYOUT>);
         const int kc = (int)(K < budget ? K : budget);
         hipLaunchKernelGGL((mam_bwd_x_kernel<LAYOUT>), dim3((unsigned)N), dim3(NT_X),
