@@ -40,8 +40,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch at the headline shape from the FETCH_SIZE / WRITE_SIZE counters, each scaled
 # by what the same counter reads for the plain 64 MiB copy made before the warm-up
 # (profiles/hbm_traffic_headline_n256_k4096_m4096.md)
-FORWARD_TRAFFIC_BYTES = {"mam_fwd_sx_kernel": 138.5e6, "mam_fwd_merge_kernel": 146.3e6}
-BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 89.7e6}
+FORWARD_TRAFFIC_BYTES = {"mam_fwd_sx_kernel": 138.7e6, "mam_fwd_merge_kernel": 145.4e6}
+BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 90.7e6}
 
 WORKLOADS = ("headline", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
              "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01", "prune_csr")
