@@ -9,10 +9,12 @@
 // HBM with coalesced stores -- no zero-fill pass and no global atomics:
 //
 //   x_grad : one workgroup per batch row n; histogram over k (chunked when K floats exceed LDS).
+//            From 2048 batch rows on: 4 to 16 rows per workgroup, the lanes of a wave spread over them.
 //   w_grad : one workgroup per R consecutive output neurons x KC consecutive k.  For the (M,K)
 //            layout R = 4 so a slab is 4 whole rows of the weight gradient (64 KiB: two
 //            workgroups per CU); for the (K,M) layout R = 32 so that every stored row segment is
-//            128 bytes.
+//            128 bytes.  From 2048 batch rows on, (M,K): up to 16 neurons per slab and the batch shared
+//            by several workgroups per slab, which add their shares to the cleared w_grad.
 //
 // Each term is one fp32 product (operand of the reference's atomicAdd); only the order of the
 // fp32 additions differs from the reference, which is itself unordered.

@@ -11,26 +11,25 @@
 //     running extreme per issue slot.  That is 2 slots per (multiply, max, min) triple.
 //   * Indices are NOT tracked per product.  Products are consumed in groups of G = 16
 //     consecutive k; after a group, one compare + one select per extreme records the group
-//     id if the running extreme strictly improved (0.25 slot per triple).  Because the test is
-//     strict, the recorded group is the one holding the FIRST occurrence of the final extreme.
-//     Both group ids share one register (16 bits each, written with sub-dword selects), which
-//     is what lets a thread keep 32 outputs and 16 k of X operands in registers at once.
+//     id if the running extreme strictly improved.  Because the test is strict, the recorded
+//     group is the one holding the FIRST occurrence of the final extreme.
 //   * An epilogue re-reads the 16 operands of the recorded group, finds the first k whose
 //     product equals the extreme, and recomputes the value from that k.  Recomputing also
 //     removes the +0/-0 ambiguity of the hardware max/min, so values and indices are exactly
-//     those of a scalar scan in ascending k with strict comparisons.
+//     those of a scalar scan in ascending k with strict comparisons.  The selected operands can
+//     be handed to the backward (w_sel, x_sel).
 //
-// Tiling: a workgroup of 256 threads (4 waves, one per SIMD) owns a 64 x 128 tile of c.  X and
-// W tiles of 32 consecutive k are staged in LDS as [row][k] (row stride 36 floats: 16-byte
-// aligned and conflict-free for ds_read_b128 along k).  A thread owns 4 x 8 outputs, strided
-// by 16 in both directions, so that a wave's W reads cover all banks and its X reads
-// broadcast.  96 of its registers hold (max, min, packed group ids); two
-// workgroups share a CU, so each SIMD always has a second wave to issue from while the other
-// waits on LDS or on the tile barrier.  Ragged edges are handled by replicating the last row /
-// column / k on load: a replicated k duplicates an earlier product and can never win a
-// strict comparison.
+// Two tilings.  The first one below (mam_fwd_kernel) takes every layout, alignment and ragged
+// size: a workgroup of 256 threads owns a 64 x 128 tile of c; X and W tiles of 32 consecutive k
+// are staged in LDS as [row][k] (row stride 36 floats: 16-byte aligned and conflict-free for
+// ds_read_b128 along k); a thread owns 4 x 8 outputs, strided by 16 in both directions, so that
+// a wave's W reads cover all banks and its X reads broadcast.  Ragged edges are handled by
+// replicating the last row / column / k on load: a replicated k duplicates an earlier product
+// and can never win a strict comparison.  The second one (mam_fwd_sx_kernel, further down)
+// serves the module's case -- (out, in) weight, aligned rows, K a multiple of 64 -- with
+// wave-uniform batch rows whose x operands come through the scalar cache.
 //
-// Small N*M (the 256 x 4096 headline shape has only 512 tiles for 256 CUs x 2) is split
+// Small N*M (the 256 x 4096 headline shape has only 256 tiles for 256 CUs x 2) is split
 // along K; each split writes (value, group) partials and a merge kernel combines them in
 // ascending k order with the same strict comparisons before resolving indices.
 #include "mam_common.h"
