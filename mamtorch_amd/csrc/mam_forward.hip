@@ -764,6 +764,8 @@ constexpr int TILE_FLOATS = BM * KT;
 constexpr int DMA_INSTR = TILE_FLOATS / 256;          // wave-level 1 KiB loads per tile
 constexpr int DMA_PER_WAVE = DMA_INSTR / (NT / 64);
 static_assert(DMA_PER_WAVE * (NT / 64) == DMA_INSTR, "tile must split evenly over the waves");
+// the resolve scratch of the epilogue lives in the dead tiles when they are large enough
+constexpr bool RES_IN_TILES = (NT / 64) * (TJ * 128 + 8 * 64) <= TILE_FLOATS;
 }  // namespace sx
 
 typedef const __attribute__((address_space(4))) float const_f32;
@@ -916,8 +918,11 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
         // and resolves it set by set; the 64 outputs of a set share their x row.
         float *vals = tile_a + wave * (sx::TJ * 128);
         int *grps = reinterpret_cast<int *>(tile_b) + wave * (sx::TJ * 128);
-        static_assert((sx::NT / 64) * (sx::TJ * 128 + RES_WORDS) <= sx::TILE_FLOATS, "resolve scratch does not fit");
-        float *res = tile_a + (sx::NT / 64) * (sx::TJ * 128) + wave * RES_WORDS;
+        static_assert((sx::NT / 64) * (sx::TJ * 128) <= sx::TILE_FLOATS, "result stash does not fit a tile buffer");
+        static_assert(RES_WORDS == 8 * 64, "sx::RES_IN_TILES assumes this size");
+        __shared__ float res_own[sx::RES_IN_TILES ? 1 : (sx::NT / 64) * RES_WORDS];
+        float *res = sx::RES_IN_TILES ? tile_a + (sx::NT / 64) * (sx::TJ * 128) + wave * RES_WORDS
+                                      : res_own + wave * RES_WORDS;
         // From here on a wave touches only its own corner of LDS, and the LDS operations of one wave
         // complete in issue order: no workgroup barrier between parking and resolving.
         __syncthreads();
