@@ -464,6 +464,9 @@ def main():
 
     import torch
 
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()      # builds only when nothing is built yet
     from mamtorch_amd import capi
 
     if not torch.cuda.is_available():

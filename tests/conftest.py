@@ -10,6 +10,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    # the libraries are built beforehand; only a tree with nothing built gets built here
+    import __graft_entry__
+
+    __graft_entry__.ensure_built()
 
 
 def pytest_collection_modifyitems(config, items):
