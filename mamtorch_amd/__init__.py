@@ -17,5 +17,6 @@ if "mamtorch_amd.build" not in getattr(sys, "orig_argv", []):
     from . import nn  # noqa: E402
     from . import sparse  # noqa: E402
     from . import capi  # noqa: E402
+    from .nn.legacy import MAMDense  # noqa: E402  (mamtorch/__init__.py:7: backwards compatibility)
 
 __version__ = "0.1.0"

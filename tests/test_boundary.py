@@ -185,3 +185,31 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--workload", "nonsense"], capture_output=True,
                        text=True)
     assert r.returncode != 0
+
+
+def test_legacy_layers_constructors_schedules_and_names():
+    """mamtorch.nn.v1.FullyConnected, mamtorch.nn.v4.FullyConnected and mamtorch.MAMDense under their
+    reference names (mamtorch/nn/__init__.py:1-6, mamtorch/__init__.py:7)."""
+    assert mt.nn.v4.FullyConnected is mt.nn.FullyConnected
+    layer = mt.nn.v1.FullyConnected(12, 6, vcon_steps=4, init_mode="normal")
+    assert repr(layer) == "MAM@FullyConnected(in_features=12, out_features=6, bias=True, vcon_steps=4, vcon_type=linear)"
+    assert layer.weight.shape == (6, 12) and bool((layer.bias == 0).all()) and layer.beta == 1.0
+    for want in (0.75, 0.5, 0.25, 0):
+        layer.vcon_step()
+        assert layer.beta == want
+    bound = (6 / (2 + 6)) ** 0.5
+    uniform = mt.nn.v1.FullyConnected(50, 6)
+    assert float(uniform.weight.abs().max()) <= bound and uniform.beta == 0.0
+    with pytest.raises(Exception, match="not supported"):
+        mt.nn.v1.FullyConnected(4, 4, vcon_steps=2, vcon_type="cubic").vcon_step()
+    with pytest.raises(Exception, match="No argmax"):
+        uniform.update_selection_count()
+    dense = mt.MAMDense(10, 3, beta=True, beta_decay="descending-parabola", beta_epochs=4)
+    assert dense.input_features == 10 and dense.state_size == 3 and dense.beta == 1.0
+    dense.adjust_beta(2)
+    assert dense.beta == 0.75
+    dense.adjust_beta(4)
+    assert dense.beta == 0
+    asc = mt.MAMDense(10, 3, beta=True, beta_decay="ascending-parabola", beta_epochs=4)
+    asc.adjust_beta(1)
+    assert abs(asc.beta - 0.5625) < 1e-12

@@ -252,3 +252,40 @@ def test_linear_layers_swapped_for_mam_and_vit_mlp_block():
     out.sum().backward()
     assert tokens.grad is not None and block.intermediate.weight.grad is not None
     assert torch.isfinite(tokens.grad).all()
+
+
+def test_legacy_layers_against_the_oracle():
+    """nn.v1.FullyConnected and MAMDense: pure MAM output bit-exact (bias added after max + min), blended
+    output against the same expression on the oracle's MAM term, gradients of both, literal selection count."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(5, 7, 40, generator=g)
+    for make in (lambda: mt.nn.v1.FullyConnected(40, 24), lambda: mt.MAMDense(40, 24)):
+        layer = make()
+        with torch.no_grad():
+            layer.bias.copy_(torch.randn(24, generator=g))
+        w, b = layer.weight.detach().clone(), layer.bias.detach().clone()
+        layer = layer.to(dev)
+        c_ref, amax, amin = oracle.forward(x.reshape(-1, 40).numpy(), w.numpy(), oracle.W_MK, b.numpy())
+        xd = x.to(dev).requires_grad_(True)
+        y = layer(xd)
+        assert y.shape == (5, 7, 24)
+        assert_bits_equal(y.detach().cpu().numpy().reshape(-1, 24), c_ref, "legacy pure MAM output")
+        assert_index_equal(layer.argmax.cpu().numpy(), amax, "argmax")
+        grad = torch.randn(5, 7, 24, generator=g)
+        y.backward(grad.to(dev))
+        xg, wg = oracle.backward(x.reshape(-1, 40).numpy(), w.numpy(), grad.reshape(-1, 24).numpy(), amax, amin, oracle.W_MK)
+        assert np.allclose(xd.grad.cpu().numpy().reshape(-1, 40), xg, rtol=1e-5, atol=1e-6)
+        assert np.allclose(layer.weight.grad.cpu().numpy(), wg, rtol=1e-5, atol=1e-6)
+        assert np.allclose(layer.bias.grad.cpu().numpy(), grad.reshape(-1, 24).sum(0).numpy(), rtol=1e-5, atol=1e-5)
+        layer.update_selection_count()
+        zeros = np.zeros((24, 40), np.int32)
+        want_count, _ = oracle.selection_count(amax, amin, zeros, zeros, mode=0)
+        assert np.array_equal(layer.max_selection_count.cpu().numpy(), want_count)
+        assert not layer.min_selection_count.any()
+        # blended: (1 - beta) * MAM + bias + beta * MAC
+        layer.beta = 0.25
+        y2 = layer(x.to(dev)).cpu()
+        c_mam = oracle.forward(x.reshape(-1, 40).numpy(), w.numpy(), oracle.W_MK)[0]
+        want = (0.75 * torch.from_numpy(c_mam) + b.view(1, -1)).view(5, 7, 24) + 0.25 * torch.nn.functional.linear(x, w)
+        assert torch.allclose(y2, want, rtol=1e-5, atol=1e-5)
