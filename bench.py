@@ -460,7 +460,7 @@ def main():
     if args.steps is None:
         args.steps = 500 if small else 20
     if args.warmup is None:
-        args.warmup = 300 if small else 10
+        args.warmup = 300 if small else 40      # the GPU clock needs a few hundred ms of work to ramp
 
     import torch
 
