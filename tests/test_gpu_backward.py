@@ -197,3 +197,31 @@ def test_large_batch_shares_of_the_batch_add_up(shape):
     amax = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32)
     amin = torch.randint(0, min(K, 3), (N, M), generator=g, dtype=torch.int32)
     _check(x, w, grad, amax.numpy(), amin.numpy(), "large batch %s" % (shape,))
+
+
+@pytest.mark.parametrize("fork", ["0", "1"])
+def test_x_grad_on_the_second_stream_or_not(fork):
+    """With both gradients asked for, x_grad may run on a second stream of the library between two events
+    (taken by itself for large problems and under graph capture); MAM_BACKWARD_FORK forces either way.
+    The caller's stream must see both results, call after call."""
+    from mamtorch_amd import capi
+
+    os.environ["MAM_BACKWARD_FORK"] = fork
+    try:
+        dev = torch.device("cuda:0")
+        g = torch.Generator().manual_seed(5)
+        N, K, M = 96, 200, 64
+        x = torch.randn(N, K, generator=g)
+        w = torch.randn(M, K, generator=g)
+        for rep in range(3):
+            grad = torch.randn(N, M, generator=g)
+            amax = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32)
+            amin = torch.randint(0, K, (N, M), generator=g, dtype=torch.int32)
+            _check(x, w, grad, amax.numpy(), amin.numpy(), "fork=%s call %d" % (fork, rep))
+            # consumers on the caller's stream right after the call, no synchronisation in between
+            xg, wg = capi.fc_backward(x.to(dev), w.to(dev), grad.to(dev), amax.to(dev), amin.to(dev), capi.W_MK)
+            sums = (xg.double().sum() + wg.double().sum()).item()
+            xo, wo = oracle.backward(x.numpy(), w.numpy(), grad.numpy(), amax.numpy(), amin.numpy(), oracle.W_MK)
+            assert abs(sums - (xo.astype(np.float64).sum() + wo.astype(np.float64).sum())) < 1e-2
+    finally:
+        os.environ.pop("MAM_BACKWARD_FORK", None)
