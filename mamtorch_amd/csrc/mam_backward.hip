@@ -20,10 +20,6 @@
 // fp32 additions differs from the reference, which is itself unordered.
 #include "mam_common.h"
 
-#include <stdlib.h>
-
-#include <mutex>
-
 namespace mam {
 namespace bwd {
 
@@ -492,33 +488,6 @@ int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t
     return check_launch("mam_bwd_x_kernel");
 }
 
-// x_grad is bound by LDS atomics and w_grad by memory traffic, and neither depends on the other: with
-// both asked for, x_grad runs on a second stream of the library (default priority, one per device)
-// between two events, so the two kernels share the chip.  The calls that enqueue the fork and the join
-// are serialised by a mutex because the events are reused.
-struct ForkJoin {
-    hipStream_t side = nullptr;
-    hipEvent_t fork = nullptr, join = nullptr;
-    bool ok = false, tried = false;
-};
-static std::mutex fork_mutex;
-static ForkJoin fork_state[16];
-
-static ForkJoin *fork_join_for_current_device()
-{
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) { (void)hipGetLastError(); return nullptr; }
-    ForkJoin &f = fork_state[dev];
-    if (!f.tried) {
-        f.tried = true;
-        f.ok = hipStreamCreateWithFlags(&f.side, hipStreamNonBlocking) == hipSuccess &&
-               hipEventCreateWithFlags(&f.fork, hipEventDisableTiming) == hipSuccess &&
-               hipEventCreateWithFlags(&f.join, hipEventDisableTiming) == hipSuccess;
-        if (!f.ok) (void)hipGetLastError();
-    }
-    return f.ok ? &f : nullptr;
-}
-
 }  // namespace bwd
 }  // namespace mam
 
@@ -549,32 +518,16 @@ extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int6
             return bwd::launch_layout<MAM_W_MK>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, xg, wg, N, K, M, on);
         return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, xg, wg, N, K, M, on);
     };
-    // The fork and the join cost ~15 us between eager launches and next to nothing inside a captured
-    // graph: taken for large problems, and always while the caller's stream is being captured.
-    // MAM_BACKWARD_FORK=0 / 1 (environment) forces it off / on.
-    const char *fork_env = getenv("MAM_BACKWARD_FORK");
-    bool fork = false;
+    // x_grad is bound by LDS atomics and w_grad by memory traffic, and neither depends on the other
     if (x_grad && w_grad) {
-        if (fork_env && (fork_env[0] == '0' || fork_env[0] == '1')) {
-            fork = fork_env[0] == '1';
-        } else {
-            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-            if (st && hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
-            fork = N * M >= (1 << 22) || (capturing == hipStreamCaptureStatusActive && N * M >= (1 << 16));
-        }
-    }
-    if (fork) {
-        std::lock_guard<std::mutex> guard(bwd::fork_mutex);
-        bwd::ForkJoin *f = bwd::fork_join_for_current_device();
-        if (f && hipEventRecord(f->fork, st) == hipSuccess && hipStreamWaitEvent(f->side, f->fork, 0) == hipSuccess) {
-            const int rc_x = launch(x_grad, nullptr, f->side);
-            const bool joined = hipEventRecord(f->join, f->side) == hipSuccess;
+        ForkedStream fork(st, N * M);
+        if (fork.forked()) {
+            const int rc_x = launch(x_grad, nullptr, fork.side());
+            fork.join_later();
             const int rc_w = launch(nullptr, w_grad, st);
-            if (!joined || hipStreamWaitEvent(st, f->join, 0) != hipSuccess)
-                return fail(MAM_ERR_LAUNCH, "could not join the x_grad stream");
-            return rc_x != MAM_OK ? rc_x : rc_w;
+            const int rc_j = fork.join();
+            return rc_x != MAM_OK ? rc_x : (rc_w != MAM_OK ? rc_w : rc_j);
         }
-        (void)hipGetLastError();
     }
     return launch(x_grad, w_grad, st);
 }

@@ -17,6 +17,27 @@ int check_launch(const char *what);
 // Asynchronously sets `count` 32-bit words to zero with a small kernel (graph-capture safe).
 int fill_zero(void *ptr, int64_t count, hipStream_t stream);
 
+// Two independent kernels of one call side by side: the first runs on a second stream of the library
+// (default priority, one per device) between a fork and a join event on the caller's stream.
+//   ForkedStream fork(st, units);      // decides; fork.side() is `st` itself when not forked
+//   launch A on fork.side(); fork.join_later(); launch B on st; rc = fork.join();
+// Between eager launches the two events cost ~15 us, inside a captured graph next to nothing: the fork
+// is taken from 2^22 `units` (outputs of the call) on, and from 2^16 on while `st` is being captured.
+// MAM_BACKWARD_FORK=0 / 1 (environment) forces it off / on.  The enqueue sequences of concurrent
+// callers are serialised (the events are reused), so an object of this class holds a lock while forked.
+class ForkedStream {
+public:
+    ForkedStream(hipStream_t st, int64_t units);
+    ~ForkedStream();
+    hipStream_t side() const { return side_; }
+    bool forked() const { return forked_; }
+    void join_later();   // after the last launch on side(): records the join event
+    int join();          // after the launches on the caller's stream: it waits for the side stream
+private:
+    hipStream_t st_, side_;
+    bool forked_, recorded_;
+};
+
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 constexpr int kNumXCD = 8;   // MI355X: 8 accelerator complex dies, each with its own L2

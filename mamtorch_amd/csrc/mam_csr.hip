@@ -487,9 +487,12 @@ extern "C" int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *c
     if (!x || !crow || !grad || !argmax || !argmin) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
     if (ldx < K) return fail(MAM_ERR_INVALID_ARGUMENT, "ldx smaller than K");
     if (handed) {
+        // the two kernels are independent: side by side where that pays (see ForkedStream)
+        ForkedStream fork(st, (x_grad && val_grad) ? N * M : 0);
         if (x_grad) {
-            rc = bwd::x_grad_from_selected(grad, argmax, argmin, w_sel, x_grad, N, K, M, st);
+            rc = bwd::x_grad_from_selected(grad, argmax, argmin, w_sel, x_grad, N, K, M, fork.side());
             if (rc != MAM_OK) return rc;
+            fork.join_later();
         }
         if (val_grad) {
             const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
@@ -500,7 +503,8 @@ extern "C" int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *c
                                vec_in);
             rc = check_launch("csr_bwd_val_kernel");
         }
-        return rc;
+        const int rc_join = fork.join();
+        return rc != MAM_OK ? rc : rc_join;
     }
     static const int budget = csr::lds_budget_floats((const void *)csr::csr_bwd_kernel);
     const int kc = (int)(K < budget ? K : budget);
