@@ -261,7 +261,8 @@ def run_dense(torch, capi, lib, dev, args):
     if wl == "headline":
         out["roofline"]["traffic"] = sum(FORWARD_TRAFFIC_BYTES.values())
         out["roofline"]["traffic_by_kernel"] = FORWARD_TRAFFIC_BYTES
-        out["roofline"]["algorithmic_bytes"] = 4 * (256 * 4096 + 4096 * 4096 + 4 * 256 * 4096)
+        # x, w, c, argmax, argmin and the four hand-over planes (w_sel, x_sel)
+        out["roofline"]["algorithmic_bytes"] = 4 * (256 * 4096 + 4096 * 4096 + 8 * 256 * 4096)
     if backward:
         bwd_ms = ph["backward"]
         out["fwd_bwd_gops"] = round(triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e9, 2)
