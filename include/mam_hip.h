@@ -45,10 +45,35 @@ extern "C" {
                                  min by >=1 row, both into max_count (the module's literal rule) */
 #define MAM_COUNT_HITS 1      /* true hit counts: max_count += #argmax hits, min_count += #argmin */
 
+/* Run-time switches for mam_set_option().  Their initial values come from the environment variables of
+ * the same names (MAM_FORWARD_TILING = auto | wide, MAM_BACKWARD_FORK = 0 | 1), read once when the
+ * library is loaded. */
+#define MAM_OPT_FORWARD_TILING 0 /* which dense forward tiling serves a call                      */
+#define MAM_OPT_BACKWARD_FORK 1  /* x_grad on the library's second stream beside w_grad           */
+#define MAM_OPT_COUNT_ 2
+#define MAM_FORWARD_TILING_AUTO 0 /* wave-uniform-rows tiling where the layout allows it           */
+#define MAM_FORWARD_TILING_WIDE 1 /* every call on the general 64 x 128 tiling                     */
+#define MAM_BACKWARD_FORK_AUTO (-1) /* from 2^22 outputs on, and under stream capture from 2^16   */
+#define MAM_BACKWARD_FORK_OFF 0
+#define MAM_BACKWARD_FORK_ON 1
+
 /* Library version (major*10000 + minor*100 + patch). */
 int mam_version(void);
 const char *mam_error_string(int code);
 const char *mam_last_error(void);
+
+/*
+ * Per-device set-up for the CURRENT HIP device: raises the LDS limit of the kernels that use more than
+ * 64 KiB and creates the library's second stream (default priority) and its two events.  Idempotent and thread-safe.  Every entry point
+ * does the same on its first call on a device; a caller that records HIP graphs calls mam_init() (or
+ * any entry point once, eagerly) on that device BEFORE capturing, because streams and events must not be
+ * created inside a capture.  No counterpart in the reference, which has no per-device state.
+ */
+int mam_init(void);
+
+/* Sets a MAM_OPT_* switch for the whole process (all devices, all threads).  The reference has no
+ * run-time switches; these exist for tests and comparisons. */
+int mam_set_option(int option, int value);
 
 /*
  * Exact MAM forward with indices.

@@ -15,11 +15,16 @@ W_MK = 1
 PRUNE_MAGNITUDE = 0
 PRUNE_WEIGHT_TIMES = 1
 PRUNE_COUNT = 2
+OPT_FORWARD_TILING = 0
+OPT_BACKWARD_FORK = 1
+FORWARD_TILING_AUTO = 0
+FORWARD_TILING_WIDE = 1
+BACKWARD_FORK_AUTO = -1
 COUNT_REFERENCE = 0
 COUNT_HITS = 1
 
 EXPORTS = (
-    "mam_version", "mam_error_string", "mam_last_error",
+    "mam_version", "mam_error_string", "mam_last_error", "mam_init", "mam_set_option",
     "mam_fc_forward_workspace", "mam_fc_forward",
     "mam_fc_forward_values_workspace", "mam_fc_forward_values",
     "mam_fc_backward", "mam_selection_count",
@@ -49,6 +54,7 @@ def lib():
             fn.argtypes = [_i64, _i64, _i64]
         l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
                                      _i64, _i64, _ptr, _size, _ptr]
+        l.mam_set_option.argtypes = [_int, _int]
         l.mam_fc_forward_values.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _i64, _i64, _i64,
                                             _ptr, _size, _ptr]
         l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
@@ -114,6 +120,10 @@ def fc_forward(x, w, layout=W_KM, bias=None, workspace=None, w_sel=None, x_sel=N
                                 _p(w_sel), _p(x_sel), N, K, M, _p(workspace), 0 if workspace is None else workspace.numel(),
                                 _stream(x)))
     return c, amax, amin
+
+
+def set_option(option, value):
+    _check(lib().mam_set_option(option, value))
 
 
 def fc_forward_values(x, w, layout=W_KM, bias=None, workspace=None):

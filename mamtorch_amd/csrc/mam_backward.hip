@@ -374,16 +374,30 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
     store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, false);
 }
 
-// LDS a workgroup may use for a histogram, in floats.  gfx950 has 160 KiB per CU; above
-// 64 KiB the kernel attribute has to be raised first.
-static int lds_budget_floats(const void *kernel)
+// LDS a workgroup may use for a histogram, in floats, per device.  gfx950 has 160 KiB per CU; above
+// 64 KiB the kernel attribute has to be raised first, once per device, which the device's set-up does
+// for every kernel of this file.
+static int g_lds_floats[kMaxDevices];
+
+static int setup_device(int dev)
 {
     constexpr int kWant = 128 * 1024;
-    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kWant) == hipSuccess)
-        return kWant / 4;
-    (void)hipGetLastError();
-    return 64 * 1024 / 4;
+    const void *kernels[] = {
+        (const void *)mam_bwd_x_rows_kernel<MAM_W_MK>, (const void *)mam_bwd_x_rows_kernel<MAM_W_KM>,
+        (const void *)mam_bwd_x_kernel<MAM_W_MK>,      (const void *)mam_bwd_x_kernel<MAM_W_KM>,
+        (const void *)mam_bwd_w_kernel<MAM_W_MK>,      (const void *)mam_bwd_w_kernel<MAM_W_KM>,
+        (const void *)mam_bwd_w_vec_kernel<MAM_W_MK>,  (const void *)mam_bwd_w_vec_kernel<MAM_W_KM>,
+    };
+    bool all = true;
+    for (const void *k : kernels)
+        if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kWant) != hipSuccess) {
+            (void)hipGetLastError();
+            all = false;
+        }
+    g_lds_floats[dev] = (all ? kWant : 64 * 1024) / 4;
+    return MAM_OK;
 }
+static DeviceHookRegistration g_registration(setup_device);
 
 template <int LAYOUT>
 static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ldw, const float *grad,
@@ -391,6 +405,10 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
                          float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
 {
     int rc = MAM_OK;
+    const int dev = ensure_device();
+    if (dev < 0) return dev;
+    const int lds_cap = g_lds_floats[dev];
+    const int cus = num_cus();
     const bool x_rows = N >= 2048 && K * 16 <= 64 * 1024 && (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
                         ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) &&
                         ((uintptr_t)w_sel % 16 == 0);
@@ -399,16 +417,13 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         int log2r = 2;
         while (log2r < 4 && ((int64_t)2 << log2r) * K * 4 <= 64 * 1024) ++log2r;
         const int R = 1 << log2r;
-        static const int ok = lds_budget_floats((const void *)mam_bwd_x_rows_kernel<LAYOUT>);
-        (void)ok;
         hipLaunchKernelGGL((mam_bwd_x_rows_kernel<LAYOUT>), dim3((unsigned)ceil_div(N, R)), dim3(NT_W),
                            (size_t)R * K * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M, x_grad,
                            (int)N, (int)K, (int)M, log2r);
         rc = check_launch("mam_bwd_x_rows_kernel");
         if (rc != MAM_OK) return rc;
     } else if (x_grad) {
-        static const int budget = lds_budget_floats((const void *)mam_bwd_x_kernel<LAYOUT>);
-        const int kc = (int)(K < budget ? K : budget);
+        const int kc = (int)(K < lds_cap ? K : lds_cap);
         hipLaunchKernelGGL((mam_bwd_x_kernel<LAYOUT>), dim3((unsigned)N), dim3(NT_X),
                            (size_t)kc * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M,
                            x_grad, (int)K, (int)M, kc);
@@ -418,8 +433,6 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
     if (w_grad) {
         // (M,K): 4 whole-K rows in 64 KiB, so two workgroups share a CU.  (K,M): 32 columns x
         // 1024 k in 128 KiB.
-        static const int big = lds_budget_floats((const void *)mam_bwd_w_kernel<LAYOUT>);
-        static const int big2 = lds_budget_floats((const void *)mam_bwd_w_vec_kernel<LAYOUT>);
         const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
                            ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)x_sel % 16 == 0) && (N * M % 4 == 0);
         int log2r = LAYOUT == MAM_W_MK ? 2 : 5;
@@ -431,7 +444,6 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         if (large_batch)
             while (log2r < 4 && ((int64_t)2 << log2r) * ((K + 3) / 4 * 4) * 4 <= 64 * 1024) ++log2r;
         const int R = 1 << log2r;
-        const int lds_cap = big < big2 ? big : big2;
         const int budget = LAYOUT == MAM_W_MK ? (R * 4096 < lds_cap ? R * 4096 : lds_cap) : lds_cap;
         int kc = budget / R;
         if (K < kc) kc = (int)((K + 3) / 4 * 4);
@@ -440,7 +452,7 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         const int vec_out = (K % 4 == 0) && ((uintptr_t)w_grad % 16 == 0);
         if (vec_in) {
             // slabs per workgroup: enough workgroups for two per CU, the rest goes into pipelining
-            int tpw = (int)(mtiles * ktiles / (2 * kNumCU));
+            int tpw = (int)(mtiles * ktiles / (2 * cus));
             if (tpw < 1) tpw = 1;
             if (tpw > 8) tpw = 8;
             // shares of the batch per slab: two rounds of as many workgroups as fit the chip (LDS, threads)
@@ -449,7 +461,7 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
                 int64_t per_cu = (160 * 1024) / ((int64_t)R * kc * 4);
                 if (per_cu > 2048 / NT_W) per_cu = 2048 / NT_W;
                 if (per_cu < 1) per_cu = 1;
-                shares = (2 * per_cu * kNumCU + mtiles * ktiles / 2) / (mtiles * ktiles);
+                shares = (2 * per_cu * cus + mtiles * ktiles / 2) / (mtiles * ktiles);
                 // a share adds a whole slab to w_grad with atomics: worth it only against >= K rows of work
                 if (shares > N / (K > 512 ? K : 512)) shares = N / (K > 512 ? K : 512);
                 if (shares > 65535) shares = 65535;
@@ -480,8 +492,9 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
 int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t *argmin, const float *w_sel,
                          float *x_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
 {
-    static const int budget = lds_budget_floats((const void *)mam_bwd_x_kernel<MAM_W_MK>);
-    const int kc = (int)(K < budget ? K : budget);
+    const int dev = ensure_device();
+    if (dev < 0) return dev;
+    const int kc = (int)(K < g_lds_floats[dev] ? K : g_lds_floats[dev]);
     hipLaunchKernelGGL((mam_bwd_x_kernel<MAM_W_MK>), dim3((unsigned)N), dim3(NT_X), (size_t)kc * sizeof(float),
                        st, (const float *)nullptr, (int64_t)0, grad, argmax, argmin, w_sel, N * M, x_grad, (int)K,
                        (int)M, kc);

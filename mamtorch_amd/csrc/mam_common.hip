@@ -4,6 +4,9 @@
 #include <stdarg.h>
 #include <stdlib.h>
 
+#include <string.h>
+
+#include <atomic>
 #include <mutex>
 
 namespace mam {
@@ -43,72 +46,125 @@ int fill_zero(void *ptr, int64_t count, hipStream_t stream)
 }
 
 namespace {
-struct SideStream {
-    hipStream_t stream = nullptr;
+struct DeviceState {
+    std::mutex lock;             // set-up of this device, and its fork/join sequences
+    std::atomic<int> ready{0};   // 1 once every hook has run
+    int rc = MAM_OK;
+    std::atomic<int> cus{0};     // compute units, 0 = not asked yet
+    hipStream_t stream = nullptr;   // the library's second stream (default priority)
     hipEvent_t fork = nullptr, join = nullptr;
-    bool ok = false, tried = false;
+    bool side_ok = false;
 };
-std::mutex side_mutex;
-SideStream side_streams[16];
+DeviceState g_devices[kMaxDevices];
 
-SideStream *side_stream_of_current_device()
+constexpr int kMaxHooks = 16;
+DeviceHook g_hooks[kMaxHooks];
+int g_num_hooks = 0;
+
+int env_choice(const char *name, int fallback)
 {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) {
-        (void)hipGetLastError();
-        return nullptr;
-    }
-    SideStream &s = side_streams[dev];
-    if (!s.tried) {
-        s.tried = true;
-        s.ok = hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) == hipSuccess &&
-               hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) == hipSuccess &&
-               hipEventCreateWithFlags(&s.join, hipEventDisableTiming) == hipSuccess;
-        if (!s.ok) (void)hipGetLastError();
-    }
-    return s.ok ? &s : nullptr;
+    const char *v = getenv(name);
+    if (!v || !v[0]) return fallback;
+    if (strcmp(v, "wide") == 0) return MAM_FORWARD_TILING_WIDE;
+    if (strcmp(v, "auto") == 0) return fallback;
+    return atoi(v);
 }
+// initial values from the environment, read once when the library is loaded
+std::atomic<int> g_options[MAM_OPT_COUNT_] = {
+    {env_choice("MAM_FORWARD_TILING", MAM_FORWARD_TILING_AUTO)},
+    {env_choice("MAM_BACKWARD_FORK", MAM_BACKWARD_FORK_AUTO)},
+};
 }  // namespace
 
-ForkedStream::ForkedStream(hipStream_t st, int64_t units) : st_(st), side_(st), forked_(false), recorded_(false)
+DeviceHookRegistration::DeviceHookRegistration(DeviceHook fn)
+{
+    if (g_num_hooks < kMaxHooks) g_hooks[g_num_hooks++] = fn;
+}
+
+int option(int which) { return g_options[which].load(std::memory_order_relaxed); }
+
+int ensure_device()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(MAM_ERR_LAUNCH, "no current HIP device");
+    }
+    if (dev < 0 || dev >= kMaxDevices) return fail(MAM_ERR_UNSUPPORTED, "device index %d beyond %d", dev, kMaxDevices - 1);
+    DeviceState &d = g_devices[dev];
+    if (d.ready.load(std::memory_order_acquire)) return d.rc == MAM_OK ? dev : d.rc;
+    std::lock_guard<std::mutex> hold(d.lock);
+    if (!d.ready.load(std::memory_order_relaxed)) {
+        d.side_ok = hipStreamCreateWithFlags(&d.stream, hipStreamNonBlocking) == hipSuccess &&
+                    hipEventCreateWithFlags(&d.fork, hipEventDisableTiming) == hipSuccess &&
+                    hipEventCreateWithFlags(&d.join, hipEventDisableTiming) == hipSuccess;
+        if (!d.side_ok) (void)hipGetLastError();
+        for (int i = 0; i < g_num_hooks && d.rc == MAM_OK; ++i) d.rc = g_hooks[i](dev);
+        d.ready.store(1, std::memory_order_release);
+    }
+    return d.rc == MAM_OK ? dev : d.rc;
+}
+
+int num_cus()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return kNumCU;
+    }
+    int cus = g_devices[dev].cus.load(std::memory_order_relaxed);
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+            (void)hipGetLastError();
+            cus = kNumCU;
+        }
+        g_devices[dev].cus.store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
+ForkedStream::ForkedStream(hipStream_t st, int64_t units)
+    : st_(st), side_(st), dev_(-1), forked_(false), recorded_(false)
 {
     if (units <= 0) return;
-    const char *env = getenv("MAM_BACKWARD_FORK");
+    const int choice = option(MAM_OPT_BACKWARD_FORK);
     bool want;
-    if (env && (env[0] == '0' || env[0] == '1')) {
-        want = env[0] == '1';
+    if (choice == MAM_BACKWARD_FORK_OFF || choice == MAM_BACKWARD_FORK_ON) {
+        want = choice == MAM_BACKWARD_FORK_ON;
     } else {
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
         if (st && hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
         want = units >= (1 << 22) || (capturing == hipStreamCaptureStatusActive && units >= (1 << 16));
     }
     if (!want) return;
-    side_mutex.lock();
-    SideStream *s = side_stream_of_current_device();
-    if (s && hipEventRecord(s->fork, st) == hipSuccess && hipStreamWaitEvent(s->stream, s->fork, 0) == hipSuccess) {
-        side_ = s->stream;
+    const int dev = ensure_device();
+    if (dev < 0 || !g_devices[dev].side_ok) return;
+    DeviceState &d = g_devices[dev];
+    d.lock.lock();
+    if (hipEventRecord(d.fork, st) == hipSuccess && hipStreamWaitEvent(d.stream, d.fork, 0) == hipSuccess) {
+        side_ = d.stream;
+        dev_ = dev;
         forked_ = true;
         return;
     }
     (void)hipGetLastError();
-    side_mutex.unlock();
+    d.lock.unlock();
 }
 
 void ForkedStream::join_later()
 {
     if (!forked_ || recorded_) return;
-    SideStream *s = side_stream_of_current_device();
-    recorded_ = s && hipEventRecord(s->join, side_) == hipSuccess;
+    recorded_ = hipEventRecord(g_devices[dev_].join, side_) == hipSuccess;
 }
 
 int ForkedStream::join()
 {
     if (!forked_) return MAM_OK;
     join_later();
-    SideStream *s = side_stream_of_current_device();
-    const bool ok = recorded_ && s && hipStreamWaitEvent(st_, s->join, 0) == hipSuccess;
+    DeviceState &d = g_devices[dev_];
+    const bool ok = recorded_ && hipStreamWaitEvent(st_, d.join, 0) == hipSuccess;
     forked_ = false;
-    side_mutex.unlock();
+    d.lock.unlock();
     return ok ? MAM_OK : fail(MAM_ERR_LAUNCH, "could not join the library's second stream");
 }
 
@@ -119,7 +175,20 @@ ForkedStream::~ForkedStream()
 
 }  // namespace mam
 
-extern "C" int mam_version(void) { return 100; }
+extern "C" int mam_version(void) { return 200; }
+
+extern "C" int mam_init(void)
+{
+    const int dev = mam::ensure_device();
+    return dev < 0 ? dev : MAM_OK;
+}
+
+extern "C" int mam_set_option(int option, int value)
+{
+    if (option < 0 || option >= MAM_OPT_COUNT_) return mam::fail(MAM_ERR_INVALID_ARGUMENT, "unknown option %d", option);
+    mam::g_options[option].store(value, std::memory_order_relaxed);
+    return MAM_OK;
+}
 
 extern "C" const char *mam_last_error(void) { return mam::g_last_error; }
 

@@ -389,22 +389,31 @@ __global__ __launch_bounds__(NT) void csr_bwd_val_kernel(
     }
 }
 
-// Lets `kernel` take `bytes` of dynamic LDS (more than the 64 KiB a launch gets by default).
-static int allow_lds(const void *kernel, int bytes)
-{
-    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e != hipSuccess) (void)hipGetLastError();
-    return e == hipSuccess;
-}
+// Once per device: the forward kernels park 7 planes of results per workgroup in dynamic LDS (more than
+// the 64 KiB a launch gets by default), and the fallback backward keeps up to 128 KiB of histogram.
+static int g_bwd_lds_floats[kMaxDevices];
 
-static int lds_budget_floats(const void *kernel)
+static int setup_device(int dev)
 {
+    bool ok = hipFuncSetAttribute((const void *)csr_fwd_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  7 * ROWS * 64 * 4) == hipSuccess;
+    ok = hipFuncSetAttribute((const void *)csr_fwd_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                             7 * ROWS * 256 * 4) == hipSuccess && ok;
+    if (!ok) {
+        (void)hipGetLastError();
+        return fail(MAM_ERR_LAUNCH, "could not raise the LDS limit of the CSR forward kernels");
+    }
     constexpr int kWant = 128 * 1024;
-    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kWant) == hipSuccess)
-        return kWant / 4;
-    (void)hipGetLastError();
-    return 64 * 1024 / 4;
+    if (hipFuncSetAttribute((const void *)csr_bwd_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kWant) ==
+        hipSuccess) {
+        g_bwd_lds_floats[dev] = kWant / 4;
+    } else {
+        (void)hipGetLastError();
+        g_bwd_lds_floats[dev] = 64 * 1024 / 4;
+    }
+    return MAM_OK;
 }
+static DeviceHookRegistration g_registration(setup_device);
 
 }  // namespace csr
 }  // namespace mam
@@ -437,6 +446,8 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
     if (!workspace || workspace_bytes < need || (uintptr_t)workspace % 16 != 0)
         return fail(MAM_ERR_WORKSPACE, "CSR forward needs %zu workspace bytes, 16-byte aligned, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
+    const int dev = ensure_device();
+    if (dev < 0) return dev;
     hipStream_t st = static_cast<hipStream_t>(stream);
     float *xT = static_cast<float *>(workspace);
     const int64_t gk = ceil_div(K, 32), gn = ceil_div(ldt, 32);
@@ -449,8 +460,6 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
                         ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)w_sel % 16 == 0) &&
                         ((uintptr_t)pos_sel % 16 == 0);
     if (N <= 64) {
-        static const int ok1 = csr::allow_lds((const void *)csr::csr_fwd_kernel<1>, 7 * csr::ROWS * 64 * 4);
-        (void)ok1;
         hipLaunchKernelGGL((csr::csr_fwd_kernel<1>), dim3((unsigned)ceil_div(M, csr::ROWS), 1u), dim3(csr::NT_F),
                            (size_t)7 * csr::ROWS * 64 * sizeof(float),
                            st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel, pos_sel, (int)N,
@@ -458,8 +467,6 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
     } else {
         const int64_t gy = ceil_div(N, 256);
         if (gy > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the CSR forward grid");
-        static const int ok4 = csr::allow_lds((const void *)csr::csr_fwd_kernel<4>, 7 * csr::ROWS * 256 * 4);
-        (void)ok4;
         hipLaunchKernelGGL((csr::csr_fwd_kernel<4>), dim3((unsigned)ceil_div(M, csr::ROWS), (unsigned)gy),
                            dim3(csr::NT_F), (size_t)7 * csr::ROWS * 256 * sizeof(float), st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel,
                            pos_sel, (int)N, (int)K, (int)M, vec_out);
@@ -506,7 +513,9 @@ extern "C" int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *c
         const int rc_join = fork.join();
         return rc != MAM_OK ? rc : rc_join;
     }
-    static const int budget = csr::lds_budget_floats((const void *)csr::csr_bwd_kernel);
+    const int dev = ensure_device();
+    if (dev < 0) return dev;
+    const int budget = csr::g_bwd_lds_floats[dev];
     const int kc = (int)(K < budget ? K : budget);
     hipLaunchKernelGGL(csr::csr_bwd_kernel, dim3((unsigned)N), dim3(csr::NT_B), (size_t)kc * sizeof(float),
                        st, x, ldx, crow, col, val, grad, argmax, argmin, x_grad, val_grad, (int)K, (int)M,

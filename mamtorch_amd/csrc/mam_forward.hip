@@ -33,6 +33,7 @@
 // along K; each split writes (value, group) partials and a merge kernel combines them in
 // ascending k order with the same strict comparisons before resolving indices.
 #include "mam_common.h"
+#include "mam_offsets.h"
 
 #include <stdlib.h>
 #include <string.h>
@@ -703,7 +704,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
         const int mb = mbase < p.M ? mbase : p.M - 1;
         const char *wrows = reinterpret_cast<const char *>(p.w + (int64_t)mb * p.ldw);
         const uint32_t ldw4 = (uint32_t)p.ldw * 4u;
-        const uint32_t last = (uint32_t)(p.M - 1 - mb) * ldw4;
+        const uint32_t last = last_row_offset(p.M, mb, 16, ldw4);
         const uint32_t mine = (uint32_t)(lane >> 3) * ldw4;
         resolve_wave(p, &vals_s[wave][0][0], &grps_s[wave][0][0], &res_s[wave][0], lane,
                      [&](int slot, int &n, int &m, bool &valid) {
@@ -719,7 +720,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
                          const uint32_t row = mine + (uint32_t)(8 * (r & 1)) * ldw4;
                          const uint32_t k4 = (uint32_t)kb * 4u;
                          xp = reinterpret_cast<const float *>(xrow + k4);
-                         wp = reinterpret_cast<const float *>(wrows + ((row < last ? row : last) + k4));
+                         wp = reinterpret_cast<const float *>(wrows + (clamped_row_offset(row, last) + k4));
                      });
     } else if (live) {
         finish<LAYOUT, ARGS>(p, n_own, m_own, vmax, vmin, gmax, gmin);
@@ -746,36 +747,40 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
 // headline time and 6 % more on the other shapes; reading the next W column ahead of its use
 // changed nothing.
 namespace sx {
-#ifndef MAM_SX_TJ
-#define MAM_SX_TJ 2
-#endif
-#ifndef MAM_SX_KT
-#define MAM_SX_KT 64
-#endif
 constexpr int BN = 32;    // batch rows per workgroup
 constexpr int NT = 512;   // threads per workgroup
 constexpr int TI = 4;     // batch rows per wave
-constexpr int TJ = MAM_SX_TJ;     // neurons per lane
-constexpr int BM = 64 * TJ;       // neurons per workgroup
-constexpr int KT = MAM_SX_KT;     // k extent of one W tile
+constexpr int KT = 64;    // k extent of one W tile
 constexpr int CHUNKS = KT / 4;    // 16-byte chunks per neuron and tile
 constexpr int RPB = 64 / KT < 1 ? 1 : 64 / KT;   // neurons per 256 bytes of LDS (all 64 banks)
-constexpr int TILE_FLOATS = BM * KT;
-constexpr int DMA_INSTR = TILE_FLOATS / 256;          // wave-level 1 KiB loads per tile
-constexpr int DMA_PER_WAVE = DMA_INSTR / (NT / 64);
-static_assert(DMA_PER_WAVE * (NT / 64) == DMA_INSTR, "tile must split evenly over the waves");
-// the resolve scratch of the epilogue lives in the dead tiles when they are large enough
-constexpr bool RES_IN_TILES = (NT / 64) * (TJ * 128 + 8 * 64) <= TILE_FLOATS;
+// TJ = neurons per lane.  2 (128 neurons per workgroup) is what the launch uses.  Measured at the
+// 256 x 4096 x 4096 shape: 1 (64 neurons per workgroup, 512 tiles, no split of K and no merge) 0.226 ms
+// against 0.217 ms for 2 with K split in two plus the merge -- the k loop with one neuron per lane is 7 %
+// slower (twice the scalar loads per product), which costs more than the merge; 4 with 32-k tiles: the
+// same time at that shape and 6 % more on the large-batch shapes.
+template <int TJ_>
+struct Cfg {
+    static constexpr int TJ = TJ_;
+    static constexpr int BM = 64 * TJ;           // neurons per workgroup
+    static constexpr int TILE_FLOATS = BM * KT;
+    static constexpr int DMA_INSTR = TILE_FLOATS / 256;          // wave-level 1 KiB loads per tile
+    static constexpr int DMA_PER_WAVE = DMA_INSTR / (NT / 64);
+    static_assert(DMA_PER_WAVE * (NT / 64) == DMA_INSTR, "tile must split evenly over the waves");
+    // the resolve scratch of the epilogue lives in the dead tiles when they are large enough
+    static constexpr bool RES_IN_TILES = (NT / 64) * (TJ * 128 + 8 * 64) <= TILE_FLOATS;
+};
+constexpr int BM_MAX = Cfg<2>::BM;
 }  // namespace sx
 
 typedef const __attribute__((address_space(4))) float const_f32;
 
-template <bool ARGS, bool SPLIT>
+template <int TJ, bool ARGS, bool SPLIT>
 __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 {
-    __shared__ __attribute__((aligned(16))) float tile_a[sx::TILE_FLOATS];
-    __shared__ __attribute__((aligned(16))) float tile_b[sx::TILE_FLOATS];
-    __shared__ uint32_t doff_s[sx::DMA_PER_WAVE * sx::NT];
+    using C = sx::Cfg<TJ>;
+    __shared__ __attribute__((aligned(16))) float tile_a[C::TILE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float tile_b[C::TILE_FLOATS];
+    __shared__ uint32_t doff_s[C::DMA_PER_WAVE * sx::NT];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -792,17 +797,17 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     const int lin = l - grp * per_group;
     const int tn = first_n + lin % gsize;
     const int tm = lin / gsize;
-    const int row0 = tn * sx::BN + sx::TI * wave, col0 = tm * sx::BM;
+    const int row0 = tn * sx::BN + sx::TI * wave, col0 = tm * C::BM;
     const int kb = split * p.k_per_split;
     const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
     const int ntiles = (ke - kb) / sx::KT;    // the host sends only whole tiles here
 
-    float vmax[sx::TI][sx::TJ], vmin[sx::TI][sx::TJ];
-    int gmax[sx::TI][sx::TJ], gmin[sx::TI][sx::TJ];
+    float vmax[sx::TI][TJ], vmin[sx::TI][TJ];
+    int gmax[sx::TI][TJ], gmin[sx::TI][TJ];
 #pragma unroll
     for (int i = 0; i < sx::TI; ++i)
 #pragma unroll
-        for (int j = 0; j < sx::TJ; ++j) {
+        for (int j = 0; j < TJ; ++j) {
             vmax[i][j] = -__builtin_inff();
             vmin[i][j] = __builtin_inff();
             gmax[i][j] = 0;
@@ -820,7 +825,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     // per-lane byte offsets of this wave's direct-to-LDS loads, kept in LDS
     const uint32_t *doff = doff_s + tid;
 #pragma unroll
-    for (int t = 0; t < sx::DMA_PER_WAVE; ++t) {
+    for (int t = 0; t < C::DMA_PER_WAVE; ++t) {
         const int inst = wave + (sx::NT / 64) * t;
         const int r = inst * (64 / sx::CHUNKS) + lane / sx::CHUNKS;   // neuron within the tile
         // the k chunk that belongs at this LDS position
@@ -833,7 +838,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 
     auto dma = [&](const char *wk, float *tile) {
 #pragma unroll
-        for (int t = 0; t < sx::DMA_PER_WAVE; ++t) {
+        for (int t = 0; t < C::DMA_PER_WAVE; ++t) {
             const int inst = wave + (sx::NT / 64) * t;
             const char *src = wk + (uint64_t)doff[t * sx::NT];
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
@@ -850,7 +855,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 #pragma unroll
                 for (int q = 0; q < G; ++q) xv[i][q] = xr[i][t * sx::KT + gg * G + q];
 #pragma unroll
-            for (int j = 0; j < sx::TJ; ++j) {
+            for (int j = 0; j < TJ; ++j) {
                 float wv[G];
 #pragma unroll
                 for (int q = 0; q < G / 4; ++q) {
@@ -904,7 +909,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 #pragma unroll
         for (int i = 0; i < sx::TI; ++i)
 #pragma unroll
-            for (int j = 0; j < sx::TJ; ++j) {
+            for (int j = 0; j < TJ; ++j) {
                 const int n = row0 + i, m = col0 + lane + 64 * j;
                 if (n < p.N && m < p.M) {
                     const int64_t o = (int64_t)n * p.M + m;
@@ -916,12 +921,12 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     } else if (ARGS) {
         // A wave parks one batch row (4 sets of 64 neurons) in its own corner of the dead tiles
         // and resolves it set by set; the 64 outputs of a set share their x row.
-        float *vals = tile_a + wave * (sx::TJ * 128);
-        int *grps = reinterpret_cast<int *>(tile_b) + wave * (sx::TJ * 128);
-        static_assert((sx::NT / 64) * (sx::TJ * 128) <= sx::TILE_FLOATS, "result stash does not fit a tile buffer");
-        static_assert(RES_WORDS == 8 * 64, "sx::RES_IN_TILES assumes this size");
-        __shared__ float res_own[sx::RES_IN_TILES ? 1 : (sx::NT / 64) * RES_WORDS];
-        float *res = sx::RES_IN_TILES ? tile_a + (sx::NT / 64) * (sx::TJ * 128) + wave * RES_WORDS
+        float *vals = tile_a + wave * (TJ * 128);
+        int *grps = reinterpret_cast<int *>(tile_b) + wave * (TJ * 128);
+        static_assert((sx::NT / 64) * (TJ * 128) <= C::TILE_FLOATS, "result stash does not fit a tile buffer");
+        static_assert(RES_WORDS == 8 * 64, "C::RES_IN_TILES assumes this size");
+        __shared__ float res_own[C::RES_IN_TILES ? 1 : (sx::NT / 64) * RES_WORDS];
+        float *res = C::RES_IN_TILES ? tile_a + (sx::NT / 64) * (TJ * 128) + wave * RES_WORDS
                                       : res_own + wave * RES_WORDS;
         // From here on a wave touches only its own corner of LDS, and the LDS operations of one wave
         // complete in issue order: no workgroup barrier between parking and resolving.
@@ -929,7 +934,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 #pragma unroll
         for (int i = 0; i < sx::TI; ++i) {
 #pragma unroll
-            for (int j = 0; j < sx::TJ; ++j) {
+            for (int j = 0; j < TJ; ++j) {
                 vals[(j * 2 + 0) * 64 + lane] = vmax[i][j];
                 vals[(j * 2 + 1) * 64 + lane] = vmin[i][j];
                 grps[(j * 2 + 0) * 64 + lane] = g0 + gmax[i][j];
@@ -942,11 +947,11 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
             const char *xrow = reinterpret_cast<const char *>(p.x + (int64_t)(nrow < p.N ? nrow : p.N - 1) * p.ldx);
             const uint32_t ldw4 = (uint32_t)p.ldw * 4u;
 #pragma unroll 1
-            for (int j = 0; j < sx::TJ; ++j) {
+            for (int j = 0; j < TJ; ++j) {
                 const int mbase = col0 + 64 * j;
                 const int mb = mbase < p.M ? mbase : p.M - 1;
                 const char *wrows = reinterpret_cast<const char *>(p.w + (int64_t)mb * p.ldw);
-                const uint32_t last = (uint32_t)(p.M - 1 - mb) * ldw4;     // neurons past M repeat the last one
+                const uint32_t last = last_row_offset(p.M, mb, 64, ldw4);   // neurons past M repeat the last one
                 const uint32_t mine = (uint32_t)(lane >> 3) * ldw4;         // slot = 8 r + lane / 8
                 resolve_wave(p, vals + j * 128, grps + j * 128, res, lane,
                              [&](int slot, int &n, int &m, bool &valid) {
@@ -960,25 +965,25 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
                                  const uint32_t row = mine + (uint32_t)(8 * r) * ldw4;
                                  const uint32_t k4 = (uint32_t)kb * 4u;
                                  xp = reinterpret_cast<const float *>(xrow + k4);
-                                 wp = reinterpret_cast<const float *>(wrows + ((row < last ? row : last) + k4));
+                                 wp = reinterpret_cast<const float *>(wrows + (clamped_row_offset(row, last) + k4));
                              });
             }
         }
     } else {
         // values only: every thread parks its 16 results in its own LDS slots so that finishing them
         // is one rolled loop (one copy of the code, no register array indexed at run time)
-        static_assert(sx::TI * sx::TJ * sx::NT <= sx::TILE_FLOATS, "result stash does not fit a tile buffer");
+        static_assert(sx::TI * TJ * sx::NT <= C::TILE_FLOATS, "result stash does not fit a tile buffer");
         float *smax = tile_a + tid, *smin = tile_b + tid;
 #pragma unroll
         for (int i = 0; i < sx::TI; ++i)
 #pragma unroll
-            for (int j = 0; j < sx::TJ; ++j) {
-                smax[(i * sx::TJ + j) * sx::NT] = vmax[i][j];
-                smin[(i * sx::TJ + j) * sx::NT] = vmin[i][j];
+            for (int j = 0; j < TJ; ++j) {
+                smax[(i * TJ + j) * sx::NT] = vmax[i][j];
+                smin[(i * TJ + j) * sx::NT] = vmin[i][j];
             }
 #pragma unroll 1
-        for (int o = 0; o < sx::TI * sx::TJ; ++o) {
-            const int n = row0 + o / sx::TJ, m = col0 + lane + 64 * (o % sx::TJ);
+        for (int o = 0; o < sx::TI * TJ; ++o) {
+            const int n = row0 + o / TJ, m = col0 + lane + 64 * (o % TJ);
             if (n < p.N && m < p.M) {
                 float hi = smax[o * sx::NT], lo = smin[o * sx::NT];
                 if (hi == 0.0f || lo == 0.0f) {
@@ -1004,7 +1009,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 static int choose_splits(int64_t N, int64_t K, int64_t M, int bn = BN, int bm = BM)
 {
     const int64_t tiles = ceil_div(N, bn) * ceil_div(M, bm);
-    const int64_t want = 2 * kNumCU;
+    const int64_t want = 2 * num_cus();
     if (tiles >= want) return 1;
     int64_t s = ceil_div(want, tiles);
     const int64_t max_by_k = K / (8 * KT);  // keep at least 256 k per split
@@ -1019,7 +1024,7 @@ static int choose_splits(int64_t N, int64_t K, int64_t M, int bn = BN, int bm = 
 static size_t workspace_bytes(int64_t N, int64_t K, int64_t M, bool args)
 {
     // whichever tiling the launch picks (it depends on alignment, unknown here): the larger need
-    const int s1 = choose_splits(N, K, M), s2 = choose_splits(N, K, M, sx::BN, sx::BM);
+    const int s1 = choose_splits(N, K, M), s2 = choose_splits(N, K, M, sx::BN, sx::BM_MAX);
     const int s = s1 > s2 ? s1 : s2;
     if (s == 1) return 0;
     return (size_t)s * (args ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float);
@@ -1048,13 +1053,13 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     p.N = (int)N; p.K = (int)K; p.M = (int)M;
     p.vec_x = (ldx % 4 == 0) && ((uintptr_t)x % 16 == 0);
     p.vec_w = (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0);
-    // The wave-uniform-rows tiling takes (M,K) weights with aligned rows and whole 32-k tiles; the
-    // environment variable MAM_FORWARD_TILING=wide keeps every shape on the first tiling (for
+    // The wave-uniform-rows tiling takes (M,K) weights with aligned rows and whole 64-k tiles; option
+    // MAM_OPT_FORWARD_TILING = MAM_FORWARD_TILING_WIDE keeps every shape on the first tiling (for
     // comparisons and tests).
-    const char *tiling = getenv("MAM_FORWARD_TILING");
     const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % sx::KT == 0) &&
-                        (ldw * sx::BM < (1ll << 30)) && !(tiling && strcmp(tiling, "wide") == 0);
-    const int bn = use_sx ? sx::BN : BN, bm = use_sx ? sx::BM : BM;
+                        (ldw * sx::BM_MAX < (1ll << 30)) &&
+                        option(MAM_OPT_FORWARD_TILING) != MAM_FORWARD_TILING_WIDE;
+    const int bn = use_sx ? sx::BN : BN, bm = use_sx ? sx::BM_MAX : BM;
     p.tiles_n = (int)ceil_div(N, bn);
     p.tiles_m = (int)ceil_div(M, bm);
     p.splits = choose_splits(N, K, M, bn, bm);
@@ -1062,8 +1067,8 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), kt) * kt);
     p.splits = (int)ceil_div(K, p.k_per_split);
     p.part = nullptr;
-    if (p.splits > 1) {
-        const size_t need = (size_t)p.splits * (ARGS ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float);
+    const size_t need = p.splits > 1 ? (size_t)p.splits * (ARGS ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float) : 0;
+    if (need > 0) {
         if (!workspace || workspace_size < need)
             return fail(MAM_ERR_WORKSPACE, "forward needs %zu workspace bytes, got %zu", need,
                         workspace ? workspace_size : (size_t)0);
@@ -1080,11 +1085,13 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
 
     const int64_t nblk = (int64_t)p.tiles_n * p.tiles_m * p.splits;
     if (nblk > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "too many tiles");
+    const int dev = ensure_device();
+    if (dev < 0) return dev;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (use_sx && p.splits > 1)
-        hipLaunchKernelGGL((mam_fwd_sx_kernel<ARGS, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (use_sx)
-        hipLaunchKernelGGL((mam_fwd_sx_kernel<ARGS, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (w_layout == MAM_W_MK)
         hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_MK, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
     else

@@ -213,3 +213,34 @@ def test_legacy_layers_constructors_schedules_and_names():
     asc = mt.MAMDense(10, 3, beta=True, beta_decay="ascending-parabola", beta_epochs=4)
     asc.adjust_beta(1)
     assert abs(asc.beta - 0.5625) < 1e-12
+
+
+def test_resolve_row_offsets_at_a_weight_beyond_4_gib(tmp_path):
+    """The 32-bit weight-row offsets of the index-resolving code (mamtorch_amd/csrc/mam_offsets.h), checked
+    by a host-only C++ program at M = 262150, ldw = 4096, where (M - 1) * ldw * 4 wraps in 32 bits."""
+    import subprocess
+
+    exe = str(tmp_path / "offsets_host")
+    subprocess.run(["g++", "-O1", "-std=c++17", os.path.join(ROOT, "tests", "offsets_host.cpp"), "-o", exe], check=True)
+    r = subprocess.run([exe], stdout=subprocess.PIPE, text=True)
+    assert r.returncode == 0, r.stdout[-2000:]
+
+
+def test_options_are_validated():
+    l = capi.lib()
+    assert l.mam_set_option(99, 0) == -1
+    assert l.mam_set_option(capi.OPT_FORWARD_TILING, capi.FORWARD_TILING_AUTO) == 0
+
+
+def test_the_reference_import_name():
+    import mamtorch
+    import mamtorch.kernel.v4.fullyconnected_fast  # noqa: F401
+    import mamtorch.nn.compat
+    import mamtorch.nn.v1.fullyconnected
+    import mamtorch.nn.v4.fullyconnected
+    import mamtorch.sparse.kernel.v1.cusparsemm  # noqa: F401
+
+    assert mamtorch.nn.FullyConnected is mt.nn.FullyConnected is mamtorch.nn.v4.fullyconnected.FullyConnected
+    assert mamtorch.nn.v1.fullyconnected.FullyConnected is mt.nn.FullyConnectedV1
+    assert mamtorch.MAMDense is mamtorch.nn.compat.MAMDense
+    assert mamtorch.kernel.v4.fullyconnected is mt.kernel.v4.fullyconnected

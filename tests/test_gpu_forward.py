@@ -21,13 +21,16 @@ def _dev():
 
 @contextlib.contextmanager
 def forward_tiling(name):
-    """MAM_FORWARD_TILING (read by the library at every call) for the calls inside the block."""
+    """Option MAM_OPT_FORWARD_TILING of the library for the calls inside the block."""
+    from mamtorch_amd import capi
+
     if name:
-        os.environ["MAM_FORWARD_TILING"] = name
+        assert name == "wide"
+        capi.set_option(capi.OPT_FORWARD_TILING, capi.FORWARD_TILING_WIDE)
     try:
         yield
     finally:
-        os.environ.pop("MAM_FORWARD_TILING", None)
+        capi.set_option(capi.OPT_FORWARD_TILING, capi.FORWARD_TILING_AUTO)
 
 
 def _run_both_layouts(x, w_mk, bias=None, what=""):
@@ -39,7 +42,7 @@ def _run_both_layouts(x, w_mk, bias=None, what=""):
     xd = x.to(dev)
     bd = None if bias is None else bias.to(dev)
     # the (M,K) layout twice: the library picks its wave-uniform-rows tiling where the shape allows it;
-    # MAM_FORWARD_TILING=wide (read at every call) keeps it on the first tiling
+    # option MAM_FORWARD_TILING_WIDE keeps it on the first tiling
     for layout, w, tiling in ((capi.W_MK, w_mk.contiguous(), None), (capi.W_MK, w_mk.contiguous(), "wide"),
                               (capi.W_KM, w_mk.T.contiguous(), None)):
         wd = w.to(dev)
@@ -314,6 +317,44 @@ def test_large_batch_inference_config4(M):
     # the (K, M) operand gives the same answer
     c2, amax2, amin2 = capi.fc_forward(xd[:2048], wd.T.contiguous(), capi.W_KM)
     assert torch.equal(c2, c[:2048]) and torch.equal(amax2, amax[:2048]) and torch.equal(amin2, amin[:2048])
+
+
+def test_large_batch_inference_config4_out16384():
+    """The largest forward of the configurations: N16384 K4096 M16384 (1.1 T triples, 3 x 1 GiB of outputs,
+    a 256 MiB weight): oracle on sampled rows (bits and indices), and on ALL rows, in slabs of 2048 rows,
+    the selected products reproduce c, max >= min, indices in range, values-only forward equal."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    N, K, M = 16384, 4096, 16384
+    g = torch.Generator().manual_seed(16384)
+    x = torch.rand(N, K, generator=g) * 2 - 1
+    w = torch.randn(M, K, generator=g) * 0.02
+    xd, wd = x.to(dev), w.to(dev)
+    assert capi.lib().mam_fc_forward_workspace(N, K, M) == 0
+    c, amax, amin = capi.fc_forward(xd, wd, capi.W_MK)
+    torch.cuda.synchronize()
+    rows = torch.arange(7, N, 1021)       # 17 rows, among them rows of the first and of the last row tile
+    rows = torch.cat([rows, torch.tensor([0, N - 1])])
+    want = oracle.forward(x[rows].numpy(), w.numpy(), oracle.W_MK)
+    assert_bits_equal(c[rows.to(dev)].cpu().numpy(), want[0], "config 4 out 16384 c")
+    assert_index_equal(amax[rows.to(dev)].cpu().numpy(), want[1], "config 4 out 16384 argmax")
+    assert_index_equal(amin[rows.to(dev)].cpu().numpy(), want[2], "config 4 out 16384 argmin")
+    del want
+    cols = torch.arange(M, device=dev)[None, :]
+    for r0 in range(0, N, 2048):
+        sl = slice(r0, r0 + 2048)
+        i1, i2 = amax[sl].long(), amin[sl].long()
+        assert int(i1.min()) >= 0 and int(i1.max()) < K and int(i2.min()) >= 0 and int(i2.max()) < K
+        pm = torch.gather(xd[sl], 1, i1) * wd[cols, i1]
+        pn = torch.gather(xd[sl], 1, i2) * wd[cols, i2]
+        assert torch.equal(pm + pn, c[sl]), "rows %d.." % r0
+        assert bool((pm >= pn).all())
+        del i1, i2, pm, pn
+    del amax, amin
+    cv = capi.fc_forward_values(xd, wd, capi.W_MK)
+    torch.cuda.synchronize()
+    assert torch.equal(cv, c)
 
 
 @pytest.mark.parametrize("shape", [(64, 784, 256), (256, 4096, 512), (70, 123, 45), (300, 2048, 200)])
