@@ -64,7 +64,8 @@ const char *mam_last_error(void);
 
 /*
  * Per-device set-up for the CURRENT HIP device: raises the LDS limit of the kernels that use more than
- * 64 KiB and creates the library's second stream (default priority) and its two events.  Idempotent and thread-safe.  Every entry point
+ * 64 KiB, creates the library's second stream (default priority) and its two events, and takes the
+ * address of the library's file-scope scratch array.  Idempotent and thread-safe.  Every entry point
  * does the same on its first call on a device; a caller that records HIP graphs calls mam_init() (or
  * any entry point once, eagerly) on that device BEFORE capturing, because streams and events must not be
  * created inside a capture.  No counterpart in the reference, which has no per-device state.
@@ -95,6 +96,25 @@ int mam_fc_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int
                    const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel,
                    float *x_sel, int64_t N, int64_t K, int64_t M,
                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * mam_fc_forward for callers that can neither allocate nor bring a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the split-K partials go to a file-scope
+ * device array of mam_fc_forward_static_limit() bytes (32 MiB) that every GPU the library runs on holds
+ * until the process ends.  No counterpart in the reference (its launcher allocates padded copies and
+ * outputs per call, mamtorch/kernel/v1/csrc/cuda/fullyconnected.cu:246-264).  Same arguments, results and
+ * errors as mam_fc_forward without `workspace`; a call whose partials exceed the limit is refused with
+ * MAM_ERR_UNSUPPORTED before anything is launched (mam_fc_forward_workspace(N, K, M) <=
+ * mam_fc_forward_static_limit() guarantees a fit; the query covers the worst alignment, so a call may fit
+ * although it says more).  It calls no allocating routine.  All calls on one GPU share that GPU's
+ * array: calls that may overlap on one GPU (different streams, different threads) race on it -- serialise
+ * them, or use mam_fc_forward with one workspace per stream.  Nothing in the array has to be cleared
+ * between calls (a call writes every word it later reads).
+ */
+size_t mam_fc_forward_static_limit(void);
+int mam_fc_forward_static(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                          const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel,
+                          float *x_sel, int64_t N, int64_t K, int64_t M, void *stream);
 
 /*
  * Values-only exact forward (no indices).  Replaces mamtorch_kernel_v4::fullyconnected_fast_cuda

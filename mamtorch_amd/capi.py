@@ -25,6 +25,7 @@ COUNT_HITS = 1
 
 EXPORTS = (
     "mam_version", "mam_error_string", "mam_last_error", "mam_init", "mam_set_option",
+    "mam_fc_forward_static_limit", "mam_fc_forward_static",
     "mam_fc_forward_workspace", "mam_fc_forward",
     "mam_fc_forward_values_workspace", "mam_fc_forward_values",
     "mam_fc_backward", "mam_selection_count",
@@ -54,6 +55,10 @@ def lib():
             fn.argtypes = [_i64, _i64, _i64]
         l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
                                      _i64, _i64, _ptr, _size, _ptr]
+        l.mam_fc_forward_static_limit.restype = _size
+        l.mam_fc_forward_static_limit.argtypes = []
+        l.mam_fc_forward_static.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
+                                            _i64, _i64, _ptr]
         l.mam_set_option.argtypes = [_int, _int]
         l.mam_fc_forward_values.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _i64, _i64, _i64,
                                             _ptr, _size, _ptr]
@@ -120,6 +125,16 @@ def fc_forward(x, w, layout=W_KM, bias=None, workspace=None, w_sel=None, x_sel=N
                                 _p(w_sel), _p(x_sel), N, K, M, _p(workspace), 0 if workspace is None else workspace.numel(),
                                 _stream(x)))
     return c, amax, amin
+
+
+def fc_forward_static(x, w, c, argmax, argmin, layout=W_KM, bias=None, w_sel=None, x_sel=None):
+    """mam_fc_forward_static into caller-provided outputs: nothing is allocated anywhere on the way (the
+    split-K partials live in the library's file-scope device array)."""
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    with torch.cuda.device(x.device):
+        _check(l.mam_fc_forward_static(_p(x), _ld(x), _p(w), _ld(w), layout, _p(bias), _p(c), _p(argmax), _p(argmin),
+                                       _p(w_sel), _p(x_sel), N, K, M, _stream(x)))
 
 
 def set_option(option, value):

@@ -1030,10 +1030,35 @@ static size_t workspace_bytes(int64_t N, int64_t K, int64_t M, bool args)
     return (size_t)s * (args ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float);
 }
 
+// ---- the entry point that allocates nothing: split-K partials in a file-scope device array ----
+// Each GPU the library runs on holds its own copy of the array until the process ends.  Its name is a
+// host-side stand-in, not a device address: the device's set-up asks the runtime for the address once,
+// and only that pointer is handed to kernels.
+constexpr size_t kStaticScratchBytes = (size_t)32 << 20;
+static __device__ __attribute__((used)) __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void *g_scratch[kMaxDevices];
+
+static int setup_device(int dev)
+{
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+        (void)hipGetLastError();
+        g_scratch[dev] = nullptr;   // mam_fc_forward_static reports it; the other entry points do not need it
+        return MAM_OK;
+    }
+    g_scratch[dev] = ptr;
+    return MAM_OK;
+}
+static DeviceHookRegistration g_registration(setup_device);
+static size_t static_scratch_bytes() { return kStaticScratchBytes; }
+static void *static_scratch_of(int dev) { return g_scratch[dev]; }
+
 template <bool ARGS>
 static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                   const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel,
-                  int64_t N, int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream)
+                  int64_t N, int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream,
+                  bool static_scratch = false)
 {
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
     if (w_layout != MAM_W_KM && w_layout != MAM_W_MK)
@@ -1068,7 +1093,12 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     p.splits = (int)ceil_div(K, p.k_per_split);
     p.part = nullptr;
     const size_t need = p.splits > 1 ? (size_t)p.splits * (ARGS ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float) : 0;
-    if (need > 0) {
+    if (static_scratch) {
+        if (need > static_scratch_bytes())
+            return fail(MAM_ERR_UNSUPPORTED,
+                        "this shape needs %zu bytes of split-K partials, the built-in scratch array holds %zu; "
+                        "use mam_fc_forward with a workspace", need, static_scratch_bytes());
+    } else if (need > 0) {
         if (!workspace || workspace_size < need)
             return fail(MAM_ERR_WORKSPACE, "forward needs %zu workspace bytes, got %zu", need,
                         workspace ? workspace_size : (size_t)0);
@@ -1087,6 +1117,10 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     if (nblk > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "too many tiles");
     const int dev = ensure_device();
     if (dev < 0) return dev;
+    if (static_scratch && need > 0) {
+        p.part = static_cast<float *>(static_scratch_of(dev));
+        if (!p.part) return fail(MAM_ERR_LAUNCH, "the built-in scratch array has no device address");
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (use_sx && p.splits > 1)
         hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
@@ -1111,8 +1145,27 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     return rc;
 }
 
+// Every word of the partials that the merge reads is written by the same call's first kernel: nothing in
+// the array has to be cleared between calls.
+static int launch_static(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout, const float *bias,
+                         float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel, int64_t N,
+                         int64_t K, int64_t M, void *stream)
+{
+    return launch<true>(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, x_sel, N, K, M, nullptr, 0, stream,
+                        true);
+}
+
 }  // namespace fwd
 }  // namespace mam
+
+extern "C" size_t mam_fc_forward_static_limit(void) { return mam::fwd::kStaticScratchBytes; }
+
+extern "C" int mam_fc_forward_static(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                                     const float *bias, float *c, int32_t *argmax, int32_t *argmin,
+                                     float *w_sel, float *x_sel, int64_t N, int64_t K, int64_t M, void *stream)
+{
+    return mam::fwd::launch_static(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, x_sel, N, K, M, stream);
+}
 
 extern "C" size_t mam_fc_forward_workspace(int64_t N, int64_t K, int64_t M)
 {

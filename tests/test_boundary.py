@@ -226,8 +226,13 @@ def test_resolve_row_offsets_at_a_weight_beyond_4_gib(tmp_path):
     assert r.returncode == 0, r.stdout[-2000:]
 
 
-def test_options_are_validated():
+def test_static_forward_limit_is_checked_on_the_host():
     l = capi.lib()
+    N, K, M = 224, 4096, 4224      # 3 ranges of K x 3 planes x N*M words = 34 MB of partials
+    assert l.mam_fc_forward_workspace(N, K, M) > l.mam_fc_forward_static_limit() >= 24 * 2 ** 20
+    one = ctypes.c_void_p(16)       # never dereferenced: the size check precedes every launch
+    assert l.mam_fc_forward_static(one, K, one, K, capi.W_MK, None, one, one, one, None, None, N, K, M, None) == -2
+    assert b"scratch" in l.mam_last_error()
     assert l.mam_set_option(99, 0) == -1
     assert l.mam_set_option(capi.OPT_FORWARD_TILING, capi.FORWARD_TILING_AUTO) == 0
 
