@@ -34,14 +34,23 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-VALU_PEAK_TFLOPS = 78.65      # 256 CU x 4 SIMD x 16 lanes x 2 (packed width) x 2.4 GHz, no FMA x2
+# Published MI355X peaks.  The vector FP32 figure (157.3 TFLOP/s) is 256 CUs x 128 fp32 lane-operations per
+# clock x 2.4 GHz with a fused multiply-add counted as two; a (max, min, x) semiring has no fused form, so
+# its yardstick counts one operation per lane and clock: 78.65 T fp32-op/s.
+VALU_PEAK_TFLOPS = 78.65
 VECTOR_FP32_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch at the headline shape from the FETCH_SIZE / WRITE_SIZE counters, each scaled
-# by what the same counter reads for the plain 64 MiB copy made before the warm-up
-# (profiles/hbm_traffic_headline_n256_k4096_m4096.md)
+# HBM bytes per launch at the headline shape.  These are CONSTANTS copied from the committed counter
+# summary named below (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, of this same command, each scaled by
+# what the same counter reads for the plain 64 MiB copy made before the warm-up); they are not measured
+# by the run that prints them.
+TRAFFIC_PROFILE = "profiles/hbm_traffic_headline_n256_k4096_m4096.md"
 FORWARD_TRAFFIC_BYTES = {"mam_fwd_sx_kernel": 138.7e6, "mam_fwd_merge_kernel": 145.4e6}
 BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.2e6, "mam_bwd_w_vec_kernel": 90.7e6}
+SELCOUNT_TRAFFIC_BYTES = {"selcount_kernel": 166.0e6}
+RAMP_MIN_CALLS = 300          # untimed phase calls before the counted warm-up: the GPU clock ramps over them
+RAMP_MIN_SECONDS = 0.3
+RAMP_MAX_SECONDS = 3.0
 
 WORKLOADS = ("headline", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
              "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01", "prune_csr")
@@ -110,6 +119,14 @@ class Layer:
                                           self.N, self.M, self.K, self.capi.COUNT_HITS, self.sp)
         assert rc == 0, self.lib.mam_last_error()
 
+    def describe(self):
+        """Which kernels the library takes for this layer's forward (asked of the library itself)."""
+        buf = ctypes.create_string_buffer(256)
+        fn = self.lib.mam_fc_forward_describe
+        fn(self._p(self.x), self.K, self._p(self.w), self.K, self.capi.W_MK, self.N, self.K, self.M,
+           0 if self.values_only else 1, buf, 256)
+        return buf.value.decode()
+
     def backward_bytes(self):
         N, K, M = self.N, self.K, self.M
         return 4 * (N * K + N * M + 2 * N * M + 2 * N * M + N * K + K * M)
@@ -148,6 +165,19 @@ def time_phases(torch, stream, phases, steps, warmup, graph=False):
     """Runs every phase once per step; returns (ms per step by the host clock, ms per phase by events).
     graph: the step is recorded once into a HIP graph and the timed steps are replays of it; the
     per-phase times then come from a second, eager pass."""
+    # Clock ramp: the same phases, untimed, whatever --warmup says (a GPU that has been idle runs its first
+    # few hundred launches at a lower clock).  Then the counted warm-up.
+    global RAMP_REPORT
+    calls, t_ramp = 0, time.perf_counter()
+    while True:
+        for _, fn in phases:
+            fn()
+        calls += len(phases)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t_ramp
+        if (calls >= RAMP_MIN_CALLS and dt >= RAMP_MIN_SECONDS) or dt >= RAMP_MAX_SECONDS:
+            break
+    RAMP_REPORT = {"ramp_launches": calls, "ramp_ms": round(dt * 1e3, 1)}
     for _ in range(warmup):
         for _, fn in phases:
             fn()
@@ -181,6 +211,9 @@ def time_phases(torch, stream, phases, steps, warmup, graph=False):
         ms = sum(e[i].elapsed_time(e[i + 1]) for e in ev) / steps
         per_phase[label] = per_phase.get(label, 0.0) + ms
     return (ms_graph if graph else (t1 - t0) * 1e3 / steps), per_phase
+
+
+RAMP_REPORT = {}
 
 
 def valu_roofline(kernel, triples, ms):
@@ -255,12 +288,12 @@ def run_dense(torch, capi, lib, dev, args):
         "phases_ms": {k: round(v, 5) for k, v in ph.items()},
         "forward_gops": round(triples / (fwd_ms * 1e-3) / 1e9, 2),
     }
-    kernel = "mam_fwd_sx_kernel<%s> + mam_fwd_merge_kernel when K is split (one forward call per layer)" % (
-        "values" if values else "args")
+    kernel = "; ".join(sorted(set(L.describe() for L in layers))) + " (one forward call per layer)"
     out["roofline"] = valu_roofline(kernel, triples, fwd_ms)
     if wl == "headline":
         out["roofline"]["traffic"] = sum(FORWARD_TRAFFIC_BYTES.values())
         out["roofline"]["traffic_by_kernel"] = FORWARD_TRAFFIC_BYTES
+        out["roofline"]["traffic_source"] = "constant from %s, not measured by this run" % TRAFFIC_PROFILE
         # x, w, c, argmax, argmin and the four hand-over planes (w_sel, x_sel)
         out["roofline"]["algorithmic_bytes"] = 4 * (256 * 4096 + 4096 * 4096 + 8 * 256 * 4096)
     if backward:
@@ -272,6 +305,15 @@ def run_dense(torch, capi, lib, dev, args):
         if wl == "headline":
             out["roofline_backward"]["traffic"] = sum(BACKWARD_TRAFFIC_BYTES.values())
             out["roofline_backward"]["traffic_by_kernel"] = BACKWARD_TRAFFIC_BYTES
+            out["roofline_backward"]["traffic_source"] = "constant from %s, not measured by this run" % TRAFFIC_PROFILE
+    if count:
+        L = layers[0]
+        # read both index arrays, read-modify-write both counter arrays once
+        out["roofline_selection_count"] = hbm_roofline("selcount_kernel (hits mode)",
+                                                       4 * (2 * L.N * L.M + 2 * L.M * L.K), ph["selection_count"])
+        out["roofline_selection_count"]["traffic"] = sum(SELCOUNT_TRAFFIC_BYTES.values())
+        out["roofline_selection_count"]["traffic_source"] = \
+            "constant from %s, not measured by this run" % TRAFFIC_PROFILE
     cpu = None
     if args.cpu_seconds > 0:
         cpu = dense_cpu_baseline(torch, shapes, args.cpu_seconds, backward)
@@ -444,7 +486,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None,
-                    help="untimed steps; the GPU clock needs ~100 launches to ramp up")
+                    help="untimed steps after the fixed clock ramp (at least %d phase calls, always run)" % RAMP_MIN_CALLS)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--workload", choices=WORKLOADS, default="headline")
     ap.add_argument("--graph", action="store_true",
@@ -461,7 +503,7 @@ def main():
     if args.steps is None:
         args.steps = 500 if small else 20
     if args.warmup is None:
-        args.warmup = 300 if small else 40      # the GPU clock needs a few hundred ms of work to ramp
+        args.warmup = 20 if small else 5
 
     import torch
 
@@ -494,6 +536,16 @@ def main():
         "data": "synthetic",
     }
     out.update(extra)
+    out.update(RAMP_REPORT)
+    props = torch.cuda.get_device_properties(dev)
+    cu_c, khz_c = ctypes.c_int(0), ctypes.c_int(0)
+    lib.mam_device_info(ctypes.byref(cu_c), ctypes.byref(khz_c))      # what the device itself reports
+    cus = int(cu_c.value) or int(props.multi_processor_count)
+    mhz = khz_c.value / 1e3
+    out["device"] = {"name": props.name, "compute_units": cus, "max_clock_mhz": mhz,
+                     "valu_peak_from_device_tflops": round(cus * 128 * mhz * 1e6 / 1e12, 2) if mhz else None,
+                     "peaks_used": {"valu_fp32_no_fma_tflops": VALU_PEAK_TFLOPS,
+                                    "vector_fp32_tflops": VECTOR_FP32_PEAK_TFLOPS, "hbm_gbs": HBM_PEAK_GBS}}
     out["cpu_baseline"] = cpu
     print(json.dumps(out))
 

@@ -72,6 +72,10 @@ const char *mam_last_error(void);
  */
 int mam_init(void);
 
+/* Compute units and maximum engine clock (kHz) of the current device, as the library's launch heuristics
+ * see them.  Either pointer may be NULL.  No counterpart in the reference. */
+int mam_device_info(int *compute_units, int *max_clock_khz);
+
 /* Sets a MAM_OPT_* switch for the whole process (all devices, all threads).  The reference has no
  * run-time switches; these exist for tests and comparisons. */
 int mam_set_option(int option, int value);
@@ -96,6 +100,16 @@ int mam_fc_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int
                    const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel,
                    float *x_sel, int64_t N, int64_t K, int64_t M,
                    void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Writes into `text` (a host buffer of `text_bytes` bytes, NUL-terminated) which kernels mam_fc_forward
+ * (with_indices != 0) or mam_fc_forward_values (with_indices == 0) would launch for these operands: the
+ * tiling, the tile grid, the number of K ranges and the bytes of partials.  The choice depends on the
+ * alignment of x and w, so the pointers are looked at but never dereferenced.  Pure host call; for bench
+ * labels and logs.  No counterpart in the reference, which has one kernel per operator.
+ */
+int mam_fc_forward_describe(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                            int64_t N, int64_t K, int64_t M, int with_indices, char *text, size_t text_bytes);
 
 /*
  * mam_fc_forward for callers that can neither allocate nor bring a workspace (code under HIP graph
@@ -168,6 +182,18 @@ int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *crow, const i
                        const float *val, const float *bias, float *c, int32_t *argmax,
                        int32_t *argmin, float *w_sel, int32_t *pos_sel, int64_t N, int64_t K,
                        int64_t M, int64_t nnz, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Checks, on the device, the CSR invariants that mam_csr_fc_forward / _backward / mam_csr_spmm take for
+ * granted (they index x, b and the outputs with col[] and crow[] unchecked, as cusparseSpMM does behind
+ * mamtorch/sparse/kernel/v1/csrc/cuda/cusparsemm_csr.cu:37-69): *status (one int32 in device memory)
+ * receives 0 when all hold, else the OR of 1: crow[0] != 0 or crow[M] != nnz, 2: crow decreasing or out of
+ * range, 4: a column index outside [0, K), 8: columns not strictly ascending within a row (the MAM forward
+ * needs ascending columns; mam_csr_spmm does not).  Asynchronous like every other call; the caller reads
+ * *status after synchronising.  No counterpart in the reference.
+ */
+int mam_csr_validate(const int64_t *crow, const int64_t *col, int64_t M, int64_t K, int64_t nnz, int *status,
+                     void *stream);
 
 /*
  * CSR-sparse MAM backward: x_grad (N,K) dense and val_grad (nnz), both fully overwritten; either may

@@ -24,12 +24,12 @@ COUNT_REFERENCE = 0
 COUNT_HITS = 1
 
 EXPORTS = (
-    "mam_version", "mam_error_string", "mam_last_error", "mam_init", "mam_set_option",
-    "mam_fc_forward_static_limit", "mam_fc_forward_static",
+    "mam_version", "mam_error_string", "mam_last_error", "mam_init", "mam_set_option", "mam_device_info",
+    "mam_fc_forward_static_limit", "mam_fc_forward_static", "mam_fc_forward_describe",
     "mam_fc_forward_workspace", "mam_fc_forward",
     "mam_fc_forward_values_workspace", "mam_fc_forward_values",
     "mam_fc_backward", "mam_selection_count",
-    "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward",
+    "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward", "mam_csr_validate",
     "mam_csr_spmm", "mam_coo_spmm",
     "mam_prune_row_offsets", "mam_prune_fill_csr", "mam_prune_apply",
 )
@@ -60,6 +60,8 @@ def lib():
         l.mam_fc_forward_static.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
                                             _i64, _i64, _ptr]
         l.mam_set_option.argtypes = [_int, _int]
+        l.mam_fc_forward_describe.argtypes = [_ptr, _i64, _ptr, _i64, _int, _i64, _i64, _i64, _int, ctypes.c_char_p,
+                                              _size]
         l.mam_fc_forward_values.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _i64, _i64, _i64,
                                             _ptr, _size, _ptr]
         l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
@@ -69,6 +71,7 @@ def lib():
                                          _i64, _i64, _i64, _i64, _ptr, _size, _ptr]
         l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                           _ptr, _i64, _i64, _i64, _i64, _ptr]
+        l.mam_csr_validate.argtypes = [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr]
         l.mam_csr_spmm.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
         l.mam_coo_spmm.argtypes = [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
         _f = ctypes.c_float
@@ -191,6 +194,18 @@ def csr_fc_forward(x, crow, col, val, M, bias=None, w_sel=None, pos_sel=None):
                                     _p(amin), _p(w_sel), _p(pos_sel), N, K, M, val.numel(), _p(ws), need,
                                     _stream(x)))
     return c, amax, amin
+
+
+def csr_validate(crow, col, K):
+    """0 when the CSR parts satisfy what the sparse kernels assume, else a mask of violations
+    (1 row-offset ends, 2 row offsets decreasing, 4 column out of range, 8 columns not ascending in a row).
+    Synchronises to read the verdict back."""
+    l = lib()
+    M = crow.numel() - 1
+    status = torch.zeros(1, dtype=torch.int32, device=crow.device)
+    with torch.cuda.device(crow.device):
+        _check(l.mam_csr_validate(_p(crow), _p(col), M, K, col.numel(), _p(status), _stream(crow)))
+    return int(status.item())
 
 
 def csr_fc_backward(x, crow, col, val, grad, argmax, argmin, w_sel=None, pos_sel=None):

@@ -183,6 +183,24 @@ extern "C" int mam_init(void)
     return dev < 0 ? dev : MAM_OK;
 }
 
+extern "C" int mam_device_info(int *compute_units, int *max_clock_khz)
+{
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return mam::fail(MAM_ERR_LAUNCH, "no current HIP device");
+    }
+    if (compute_units) *compute_units = mam::num_cus();
+    if (max_clock_khz) {
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeClockRate, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            v = 0;
+        }
+        *max_clock_khz = v;
+    }
+    return MAM_OK;
+}
+
 extern "C" int mam_set_option(int option, int value)
 {
     if (option < 0 || option >= MAM_OPT_COUNT_) return mam::fail(MAM_ERR_INVALID_ARGUMENT, "unknown option %d", option);

@@ -1054,25 +1054,28 @@ static DeviceHookRegistration g_registration(setup_device);
 static size_t static_scratch_bytes() { return kStaticScratchBytes; }
 static void *static_scratch_of(int dev) { return g_scratch[dev]; }
 
-template <bool ARGS>
-static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
-                  const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel,
-                  int64_t N, int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream,
-                  bool static_scratch = false)
+// What a call will do: the kernel parameters, which tiling serves it, and the bytes of split-K partials.
+struct Plan {
+    Params p;
+    bool use_sx;
+    size_t need;
+};
+
+static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                     const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel,
+                     int64_t N, int64_t K, int64_t M)
 {
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
     if (w_layout != MAM_W_KM && w_layout != MAM_W_MK)
         return fail(MAM_ERR_INVALID_ARGUMENT, "w_layout must be MAM_W_KM or MAM_W_MK");
     if (N == 0 || M == 0) return MAM_OK;
     if (K == 0) return fail(MAM_ERR_INVALID_ARGUMENT, "K == 0: max/min over an empty set");
-    if (!x || !w || !c || (ARGS && (!argmax || !argmin)))
-        return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
     if (ldx < K || ldw < (w_layout == MAM_W_MK ? K : M))
         return fail(MAM_ERR_INVALID_ARGUMENT, "leading dimension smaller than the row length");
     if (N > INT32_MAX / 2 || K > INT32_MAX / 2 || M > INT32_MAX / 2)
         return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
 
-    Params p;
+    Params &p = plan.p;
     p.x = x; p.ldx = ldx; p.w = w; p.ldw = ldw; p.bias = bias;
     p.c = c; p.argmax = argmax; p.argmin = argmin; p.wsel = w_sel; p.xsel = x_sel;
     p.N = (int)N; p.K = (int)K; p.M = (int)M;
@@ -1084,6 +1087,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % sx::KT == 0) &&
                         (ldw * sx::BM_MAX < (1ll << 30)) &&
                         option(MAM_OPT_FORWARD_TILING) != MAM_FORWARD_TILING_WIDE;
+    plan.use_sx = use_sx;
     const int bn = use_sx ? sx::BN : BN, bm = use_sx ? sx::BM_MAX : BM;
     p.tiles_n = (int)ceil_div(N, bn);
     p.tiles_m = (int)ceil_div(M, bm);
@@ -1092,7 +1096,32 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), kt) * kt);
     p.splits = (int)ceil_div(K, p.k_per_split);
     p.part = nullptr;
-    const size_t need = p.splits > 1 ? (size_t)p.splits * (ARGS ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float) : 0;
+    plan.need = p.splits > 1 ? (size_t)p.splits * (args ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float) : 0;
+    // the fast staging path addresses a tile with 32-bit element offsets from the tile base
+    const int64_t w_rows = (w_layout == MAM_W_MK) ? fwd::BM : fwd::KT;
+    p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30));
+    // (16 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
+    p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 25));
+    // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
+    if ((int64_t)p.k_per_split / G > 65536)
+        return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds %d per K range", (long long)K, 65536 * G);
+    return MAM_OK;
+}
+
+template <bool ARGS>
+static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                  const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel,
+                  int64_t N, int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream,
+                  bool static_scratch = false)
+{
+    Plan plan;
+    int rc = make_plan(plan, ARGS, x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, x_sel, N, K, M);
+    if (rc != MAM_OK || N == 0 || M == 0) return rc;
+    if (!x || !w || !c || (ARGS && (!argmax || !argmin)))
+        return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    Params &p = plan.p;
+    const bool use_sx = plan.use_sx;
+    const size_t need = plan.need;
     if (static_scratch) {
         if (need > static_scratch_bytes())
             return fail(MAM_ERR_UNSUPPORTED,
@@ -1104,14 +1133,6 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
                         workspace ? workspace_size : (size_t)0);
         p.part = static_cast<float *>(workspace);
     }
-    // the fast staging path addresses a tile with 32-bit element offsets from the tile base
-    const int64_t w_rows = (w_layout == MAM_W_MK) ? fwd::BM : fwd::KT;
-    p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30));
-    // (16 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
-    p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 25));
-    // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
-    if ((int64_t)p.k_per_split / G > 65536)
-        return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds %d per K range", (long long)K, 65536 * G);
 
     const int64_t nblk = (int64_t)p.tiles_n * p.tiles_m * p.splits;
     if (nblk > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "too many tiles");
@@ -1130,7 +1151,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
         hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_MK, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
     else
         hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_KM, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
-    int rc = check_launch("mam_fwd_kernel");
+    rc = check_launch("mam_fwd_kernel");
     if (rc != MAM_OK) return rc;
     if (p.splits > 1) {
         const unsigned mb = (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
@@ -1157,6 +1178,36 @@ static int launch_static(const float *x, int64_t ldx, const float *w, int64_t ld
 
 }  // namespace fwd
 }  // namespace mam
+
+extern "C" int mam_fc_forward_describe(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                                       int64_t N, int64_t K, int64_t M, int with_indices, char *text, size_t text_bytes)
+{
+    using namespace mam;
+    fwd::Plan plan;
+    const int rc = fwd::make_plan(plan, with_indices != 0, x, ldx, w, ldw, w_layout, nullptr, nullptr, nullptr,
+                                  nullptr, nullptr, nullptr, N, K, M);
+    if (rc != MAM_OK) return rc;
+    if (!text || text_bytes == 0) return fail(MAM_ERR_INVALID_ARGUMENT, "no text buffer");
+    if (N == 0 || M == 0) {
+        snprintf(text, text_bytes, "nothing to launch");
+        return MAM_OK;
+    }
+    const fwd::Params &p = plan.p;
+    const char *what = with_indices ? "args" : "values";
+    if (plan.use_sx)
+        snprintf(text, text_bytes, "mam_fwd_sx_kernel<%s%s> %d x %d tiles of 32 x 128", what, p.splits > 1 ? ", split" : "",
+                 p.tiles_n, p.tiles_m);
+    else
+        snprintf(text, text_bytes, "mam_fwd_kernel<%s, %s> %d x %d tiles of 64 x 128", w_layout == MAM_W_MK ? "(M,K)" : "(K,M)",
+                 what, p.tiles_n, p.tiles_m);
+    if (p.splits > 1) {
+        const size_t used = strlen(text);
+        snprintf(text + used, text_bytes - used, " x %d ranges of %d k + mam_fwd_merge_kernel<%s> (%zu bytes of partials)",
+                 p.splits, p.k_per_split, (with_indices && p.coop) ? "cooperative resolve" : "per-thread resolve",
+                 plan.need);
+    }
+    return MAM_OK;
+}
 
 extern "C" size_t mam_fc_forward_static_limit(void) { return mam::fwd::kStaticScratchBytes; }
 

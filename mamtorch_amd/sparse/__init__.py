@@ -7,6 +7,8 @@ operand dispatched on the sparse-CSR key).
 """
 from . import kernel
 from . import prune
-from .fullyconnected import fullyconnected, fullyconnected_backward, SparseFullyConnectedFunction, prune_to_csr
+from .fullyconnected import (fullyconnected, fullyconnected_backward, SparseFullyConnectedFunction, prune_to_csr,
+                             validate_csr)
 
-__all__ = ["kernel", "prune", "fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr"]
+__all__ = ["kernel", "prune", "fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr",
+           "validate_csr"]

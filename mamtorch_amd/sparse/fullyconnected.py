@@ -8,7 +8,8 @@ weights whose products x*0 take part in the max / min and in the first-index tie
 import torch
 from torch import Tensor
 
-__all__ = ["fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr"]
+__all__ = ["fullyconnected", "fullyconnected_backward", "SparseFullyConnectedFunction", "prune_to_csr",
+           "validate_csr"]
 
 K = torch.ops.mamtorch_kernel_sparsev1
 
@@ -55,3 +56,26 @@ def prune_to_csr(weight: Tensor, keep_mask: Tensor) -> Tensor:
     crow[1:] = torch.cumsum(counts, dim=0)
     col = mask.nonzero()[:, 1].to(torch.int64)
     return torch.sparse_csr_tensor(crow, col, weight[mask], size=tuple(weight.shape))
+
+
+def validate_csr(w_csr: Tensor) -> None:
+    """Raises ``ValueError`` unless ``w_csr`` satisfies what the sparse kernels take for granted: row offsets
+    from 0 to nnz and non-decreasing, column indices inside [0, in_features) and strictly ascending within
+    a row.  The operators themselves do not check (a check needs a device round trip per call, and
+    ``torch.sparse_csr_tensor`` builds unchecked tensors by default), so call this once on a tensor that
+    did not come from ``Tensor.to_sparse_csr()`` / ``sparse.prune`` before handing it to them: a malformed
+    tensor makes the kernels read, and the COO SpMM write, out of range."""
+    from .. import capi
+
+    if w_csr.layout != torch.sparse_csr or w_csr.dim() != 2:
+        raise ValueError("w_csr must be a 2-dimensional torch.sparse_csr tensor")
+    crow = w_csr.crow_indices().to(torch.int64).contiguous()
+    col = w_csr.col_indices().to(torch.int64).contiguous()
+    if crow.numel() != w_csr.size(0) + 1 or col.numel() != w_csr.values().numel():
+        raise ValueError("w_csr: crow_indices / col_indices / values have inconsistent lengths")
+    bad = capi.csr_validate(crow, col, w_csr.size(1))
+    if bad:
+        what = [text for bit, text in ((1, "row offsets do not run from 0 to nnz"), (2, "row offsets decrease"),
+                                       (4, "a column index is out of range"),
+                                       (8, "column indices are not strictly ascending within a row")) if bad & bit]
+        raise ValueError("w_csr is malformed: " + "; ".join(what))

@@ -103,6 +103,45 @@ def test_implicit_zero_rules():
                       bias=torch.randn(M, generator=g))
 
 
+@pytest.mark.parametrize("K", [7, 8, 19])
+def test_signed_zeros_and_ties_inside_stored_pairs(K):
+    """Fully stored rows (no implicit zero to fall back on), so every extreme is a stored entry.  The kernel
+    records the pair of consecutive entries in which an extreme last improved and settles afterwards which
+    of the two it was: zero extremes whose first occurrence is the SECOND entry of a pair (the value must
+    carry that product's sign), ties within a pair and across pairs (lowest column wins), odd row lengths
+    (the last entry is paired with itself)."""
+    M, N = 6, 12
+    g = torch.Generator().manual_seed(K)
+    crow = torch.arange(0, (M + 1) * K, K, dtype=torch.int64)
+    col = torch.arange(K, dtype=torch.int64).repeat(M)
+    w = -torch.rand(M, K, generator=g) - 0.5            # all weights negative
+    x = torch.rand(N, K, generator=g) + 0.5              # all inputs positive: every product negative ...
+    x[0, 1] = 0.0                                        # ... except zeros: -0.0 at the second entry of pair 0
+    x[1, 1] = 0.0
+    x[1, 4] = -0.0                                       # a +0.0 product later: the max stays the first zero
+    x[2, 3] = 0.0                                        # second entry of pair 1
+    x[3, 2] = 0.0                                        # first entry of pair 1
+    x[4, K - 1] = 0.0                                    # the last entry (paired with itself when K is odd)
+    x[5, 0] = -0.0                                       # +0.0 at the very first entry
+    x[5, 1] = 0.0
+    x[6] = -x[6]                                         # all products positive: the min side gets the zeros
+    x[6, 1] = 0.0
+    x[7] = -x[7]
+    x[7, K - 1] = -0.0
+    w[1] = w[0]                                          # equal rows of w: ties between neurons are no issue
+    x[8] = 1.0
+    w[2, :] = -1.0                                       # every product equal: both extremes at column 0
+    x[9] = 1.0
+    w[3, :] = -2.0
+    w[3, 1] = -1.0                                       # max at the second entry of pair 0, min tied at 0
+    x[10] = 1.0
+    w[4, :] = -1.0
+    w[4, 5] = -3.0                                       # min at the second entry of pair 2
+    w[4, 2] = -0.5                                       # max at the first entry of pair 1
+    val = w.reshape(-1).clone()
+    _forward_backward(x, w.clone(), crow, col, val, "signed zeros and ties in pairs, K=%d" % K)
+
+
 def test_first_columns_stored_and_last_missing():
     # the lowest missing column is K-1 / is 0 / lies between stored runs
     K, N = 40, 6
@@ -161,3 +200,31 @@ def test_config5_full_size_equals_dense_kernel(density):
     for got_x, got_v in ((xg, vg), (xg2, vg2)):
         assert bool(((got_x - xdg).abs() <= 1e-5 * xdg.abs() + 2.0 ** -21 * xabs).all())
         assert bool(((got_v - want_v).abs() <= 1e-5 * want_v.abs() + 2.0 ** -21 * abs_v).all())
+
+
+def test_validate_csr_names_what_is_malformed():
+    """The operators trust the index arrays; sparse.validate_csr is the explicit check."""
+    import mamtorch_amd as mt
+
+    dev = torch.device("cuda:0")
+    dense, crow, col, val = pruned_csr(37, 50, 0.2, seed=3)
+    good = torch.sparse_csr_tensor(crow.to(dev), col.to(dev), val.to(dev), size=(37, 50))
+    mt.sparse.validate_csr(good)
+    mt.sparse.validate_csr(dense.to(dev).to_sparse_csr())
+    mt.sparse.validate_csr(torch.zeros(5, 7, device=dev).to_sparse_csr())
+    col_bad = col.clone()
+    col_bad[3] = 50
+    with pytest.raises(ValueError, match="out of range"):
+        mt.sparse.validate_csr(torch.sparse_csr_tensor(crow.to(dev), col_bad.to(dev), val.to(dev), size=(37, 50)))
+    col_swapped = col.clone()
+    col_swapped[[0, 1]] = col[[1, 0]]
+    with pytest.raises(ValueError, match="ascending"):
+        mt.sparse.validate_csr(torch.sparse_csr_tensor(crow.to(dev), col_swapped.to(dev), val.to(dev), size=(37, 50)))
+    crow_bad = crow.clone()
+    crow_bad[5], crow_bad[6] = crow[6], crow[5]
+    with pytest.raises(ValueError, match="decrease"):
+        mt.sparse.validate_csr(torch.sparse_csr_tensor(crow_bad.to(dev), col.to(dev), val.to(dev), size=(37, 50)))
+    crow_short = crow.clone()
+    crow_short[-1] -= 1
+    with pytest.raises(ValueError, match="0 to nnz"):
+        mt.sparse.validate_csr(torch.sparse_csr_tensor(crow_short.to(dev), col.to(dev), val.to(dev), size=(37, 50)))
