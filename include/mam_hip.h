@@ -44,6 +44,8 @@ extern "C" {
 #define MAM_COUNT_REFERENCE 0 /* per call: +1 per (m,k) picked as max by >=1 row, +1 if picked as
                                  min by >=1 row, both into max_count (the module's literal rule) */
 #define MAM_COUNT_HITS 1      /* true hit counts: max_count += #argmax hits, min_count += #argmin */
+#define MAM_COUNT_FLAGS 2     /* per call: max_count += 1 where >=1 row picked the cell as max, min_count
+                                 likewise for min (the retired convolution modules' literal rule)        */
 
 /* Run-time switches for mam_set_option().  Their initial values come from the environment variables of
  * the same names (MAM_FORWARD_TILING = auto | wide, MAM_BACKWARD_FORK = 0 | 1), read once when the
@@ -221,6 +223,33 @@ int mam_csr_spmm(const int64_t *crow, const int64_t *col, const float *val, cons
                  float *c, int64_t R, int64_t K, int64_t C, void *stream);
 int mam_coo_spmm(const int64_t *row, const int64_t *col, const float *val, int64_t nnz, const float *b,
                  int64_t ldb, float *c, int64_t R, int64_t K, int64_t C, void *stream);
+
+/*
+ * out (N, M) = (alpha * mam_out + beta * mac_out) + bias, each an (N, M) contiguous fp32 array (out may
+ * alias mam_out or mac_out), bias (M) or NULL: the vanishing-contribution blend of the module
+ * (mamtorch/nn/v4/fullyconnected.py:190-198) in one pass, in the reference's rounding order (two
+ * products, their sum, then the bias; nothing fused).
+ */
+int mam_blend(const float *mam_out, const float *mac_out, const float *bias, float alpha, float beta, float *out,
+              int64_t N, int64_t M, void *stream);
+
+/*
+ * MAM convolution as the MAM fully-connected kernel over gathered windows.  x is (B, C, H, W) contiguous
+ * (a 1-D convolution has H = k1 = s1 = 1), windows are k1 x k2 with strides s1, s2 and no padding (the
+ * caller pads, as the reference's modules do), output positions L1 = (H - k1) / s1 + 1, L2 likewise.
+ *   mam_im2col : cols (B * L1 * L2, k2 * k1 * C) contiguous; cols[(b, l1, l2), (j2 * k1 + j1) * C + c] =
+ *                x[b, c, l1 * s1 + j1, l2 * s2 + j2].  The column order is the index order of the reference's
+ *                retired kernels (mamtorch/kernel/backup/mamconv1d_forward.txt:128: arg = position * C +
+ *                channel; mamconv2d_forward.txt with the window column outermost), so mam_fc_forward on
+ *                (cols, weight reordered to (F, k2 * k1 * C)) yields their Y, argmax and argmin.
+ *   mam_col2im : the adjoint, x_grad (B, C, H, W) fully overwritten = sum over the windows covering each cell
+ *                of cols_grad; replaces the input-gradient half of mamconv1d/2d_backward
+ *                (mamtorch/kernel/backup/mamconv1d_backward.txt).  No atomics; fixed summation order.
+ */
+int mam_im2col(const float *x, float *cols, int64_t B, int64_t C, int64_t H, int64_t W, int64_t k1, int64_t k2,
+               int64_t s1, int64_t s2, void *stream);
+int mam_col2im(const float *cols_grad, float *x_grad, int64_t B, int64_t C, int64_t H, int64_t W, int64_t k1,
+               int64_t k2, int64_t s1, int64_t s2, void *stream);
 
 /*
  * Pruning of a dense weight w (M,K), row stride ldw, and its compaction to CSR.  An entry is pruned when

@@ -22,6 +22,7 @@ FORWARD_TILING_WIDE = 1
 BACKWARD_FORK_AUTO = -1
 COUNT_REFERENCE = 0
 COUNT_HITS = 1
+COUNT_FLAGS = 2
 
 EXPORTS = (
     "mam_version", "mam_error_string", "mam_last_error", "mam_init", "mam_set_option", "mam_device_info",
@@ -31,6 +32,7 @@ EXPORTS = (
     "mam_fc_backward", "mam_selection_count",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward", "mam_csr_validate",
     "mam_csr_spmm", "mam_coo_spmm",
+    "mam_blend", "mam_im2col", "mam_col2im",
     "mam_prune_row_offsets", "mam_prune_fill_csr", "mam_prune_apply",
 )
 
@@ -71,6 +73,9 @@ def lib():
                                          _i64, _i64, _i64, _i64, _ptr, _size, _ptr]
         l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                           _ptr, _i64, _i64, _i64, _i64, _ptr]
+        l.mam_blend.argtypes = [_ptr, _ptr, _ptr, ctypes.c_float, ctypes.c_float, _ptr, _i64, _i64, _ptr]
+        l.mam_im2col.argtypes = [_ptr, _ptr] + [_i64] * 8 + [_ptr]
+        l.mam_col2im.argtypes = [_ptr, _ptr] + [_i64] * 8 + [_ptr]
         l.mam_csr_validate.argtypes = [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr]
         l.mam_csr_spmm.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
         l.mam_coo_spmm.argtypes = [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]

@@ -14,6 +14,9 @@
 // accumulate duplicate indices, and both statements write max_selection_count, so per call a cell
 // gains 1 if any batch row picked it as argmax plus 1 if any row picked it as argmin.  The fields
 // are flags (LDS atomic or) and max_count receives flag(max) + flag(min); min_count is untouched.
+// MAM_COUNT_FLAGS: the same flags, max and min apart (max_count += flag(max), min_count += flag(min)):
+// the literal rule of the retired convolution modules (mamtorch/nn/backup/mamconv1d.txt:84-103), whose two
+// advanced-index "+= 1" statements write the two counters.
 #include "mam_common.h"
 
 namespace mam {
@@ -161,10 +164,10 @@ extern "C" int mam_selection_count(const int32_t *argmax, const int32_t *argmin,
 {
     using namespace mam;
     if (N < 0 || M < 0 || K < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
-    if (mode != MAM_COUNT_REFERENCE && mode != MAM_COUNT_HITS)
+    if (mode != MAM_COUNT_REFERENCE && mode != MAM_COUNT_HITS && mode != MAM_COUNT_FLAGS)
         return fail(MAM_ERR_INVALID_ARGUMENT, "unknown selection-count mode %d", mode);
     if (N == 0 || M == 0 || K == 0) return MAM_OK;
-    if (!argmax || !argmin || !max_count || (mode == MAM_COUNT_HITS && !min_count))
+    if (!argmax || !argmin || !max_count || (mode != MAM_COUNT_REFERENCE && !min_count))
         return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
     if (N > INT32_MAX / 2 || K > INT32_MAX / 2 || M > INT32_MAX / 2)
         return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
@@ -181,7 +184,11 @@ extern "C" int mam_selection_count(const int32_t *argmax, const int32_t *argmin,
                     (mode == MAM_COUNT_REFERENCE || (uintptr_t)min_count % 16 == 0);
     const int vec_in = (M % 4 == 0) && ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0);
     const dim3 grid((unsigned)ceil_div(M, R), (unsigned)ktiles);
-    if (mode == MAM_COUNT_HITS)
+    if (mode == MAM_COUNT_FLAGS)
+        hipLaunchKernelGGL(selcount::count_kernel<MAM_COUNT_FLAGS>, grid, dim3(selcount::NT_H),
+                           (size_t)R * kc * 4, st, argmax, argmin, max_count, min_count, (int)N, (int)M,
+                           (int)K, log2r, kc, vec, vec_in);
+    else if (mode == MAM_COUNT_HITS)
         hipLaunchKernelGGL(selcount::count_kernel<MAM_COUNT_HITS>, grid, dim3(selcount::NT_H),
                            (size_t)R * kc * 4, st, argmax, argmin, max_count, min_count, (int)N, (int)M,
                            (int)K, log2r, kc, vec, vec_in);

@@ -234,6 +234,62 @@ void selection_count(const at::Tensor &argmax, const at::Tensor &argmin, at::Ten
              "mam_selection_count");
 }
 
+// ---- module helpers: the MAC blend, and the window gather / scatter behind the MAM convolutions ----
+at::Tensor blend(const at::Tensor &mam, const at::Tensor &mac, const c10::optional<at::Tensor> &bias, double alpha,
+                 double beta)
+{
+    check_f32_2d(mam, "mam");
+    check_f32_2d(mac, "mac");
+    TORCH_CHECK(mam.sizes() == mac.sizes(), "mam and mac must have the same shape");
+    check_same_device(mam, mac, "mac");
+    const int64_t N = mam.size(0), M = mam.size(1);
+    if (bias.has_value() && bias->defined()) {
+        TORCH_CHECK(bias->is_cuda() && bias->scalar_type() == at::kFloat && bias->dim() == 1 && bias->size(0) == M &&
+                        bias->is_contiguous(),
+                    "bias must be a contiguous float32 GPU vector of out_features elements");
+        check_same_device(mam, *bias, "bias");
+    }
+    const c10::DeviceGuard guard(mam.device());
+    const at::Tensor a = mam.contiguous(), b = mac.contiguous();
+    auto out = at::empty({N, M}, mam.options());
+    check_rc(mam_blend(a.data_ptr<float>(), b.data_ptr<float>(), bias_ptr(bias), (float)alpha, (float)beta,
+                       out.data_ptr<float>(), N, M, current_stream(mam)),
+             "mam_blend");
+    return out;
+}
+
+at::Tensor im2col(const at::Tensor &x, int64_t k1, int64_t k2, int64_t s1, int64_t s2)
+{
+    TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kFloat && x.dim() == 4, "x must be a float32 GPU tensor (B, C, H, W)");
+    TORCH_CHECK(k1 >= 1 && k2 >= 1 && s1 >= 1 && s2 >= 1, "window and stride must be positive");
+    TORCH_CHECK(x.size(2) >= k1 && x.size(3) >= k2, "the window is larger than the input");
+    const c10::DeviceGuard guard(x.device());
+    const at::Tensor xc = x.contiguous();
+    const int64_t B = x.size(0), C = x.size(1), H = x.size(2), W = x.size(3);
+    const int64_t L1 = (H - k1) / s1 + 1, L2 = (W - k2) / s2 + 1;
+    auto cols = at::empty({B * L1 * L2, k2 * k1 * C}, x.options());
+    if (cols.numel() > 0)
+        check_rc(mam_im2col(xc.data_ptr<float>(), cols.data_ptr<float>(), B, C, H, W, k1, k2, s1, s2, current_stream(x)),
+                 "mam_im2col");
+    return cols;
+}
+
+at::Tensor col2im(const at::Tensor &cols, int64_t B, int64_t C, int64_t H, int64_t W, int64_t k1, int64_t k2,
+                  int64_t s1, int64_t s2)
+{
+    check_f32_2d(cols, "cols");
+    TORCH_CHECK(k1 >= 1 && k2 >= 1 && s1 >= 1 && s2 >= 1 && H >= k1 && W >= k2, "bad window geometry");
+    const int64_t L1 = (H - k1) / s1 + 1, L2 = (W - k2) / s2 + 1;
+    TORCH_CHECK(cols.size(0) == B * L1 * L2 && cols.size(1) == k2 * k1 * C, "cols does not match the geometry");
+    const c10::DeviceGuard guard(cols.device());
+    const at::Tensor cc = cols.contiguous();
+    auto xg = at::empty({B, C, H, W}, cols.options());
+    if (xg.numel() > 0)
+        check_rc(mam_col2im(cc.data_ptr<float>(), xg.data_ptr<float>(), B, C, H, W, k1, k2, s1, s2, current_stream(cols)),
+                 "mam_col2im");
+    return xg;
+}
+
 // ---- CSR-sparse MAM: w_csr is the pruned weight (out_features, in_features) ----
 struct CsrParts { at::Tensor crow, col, val; };
 
@@ -397,6 +453,9 @@ TORCH_LIBRARY(mamtorch_kernel_v4, m)
     m.def("fullyconnected_fast_wt(Tensor a, Tensor weight, Tensor? bias) -> Tensor");
     m.def("fullyconnected_wt_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin, Tensor? sel) -> Tensor[]");
     m.def("selection_count(Tensor argmax, Tensor argmin, Tensor(a!) max_count, Tensor(b!) min_count, int mode) -> ()");
+    m.def("blend(Tensor mam, Tensor mac, Tensor? bias, float alpha, float beta) -> Tensor");
+    m.def("im2col(Tensor x, int k1, int k2, int s1, int s2) -> Tensor");
+    m.def("col2im(Tensor cols, int B, int C, int H, int W, int k1, int k2, int s1, int s2) -> Tensor");
 }
 
 TORCH_LIBRARY(mamtorch_kernel_sparsev1, m)
@@ -424,6 +483,9 @@ TORCH_LIBRARY_IMPL(mamtorch_kernel_v4, CUDA, m)
     m.impl("fullyconnected_fast_wt", &fullyconnected_fast_wt);
     m.impl("fullyconnected_wt_backward", &fullyconnected_wt_backward);
     m.impl("selection_count", &selection_count);
+    m.impl("blend", &blend);
+    m.impl("im2col", &im2col);
+    m.impl("col2im", &col2im);
 }
 
 // The dense operand decides the key for mixed dense / sparse-CSR arguments only when the sparse

@@ -1,0 +1,91 @@
+"""Operators behind the module-level extras (no upstream operator names): the vanishing-contribution
+blend of ``FullyConnected`` (mamtorch/nn/v4/fullyconnected.py:190-198) as one kernel, and the window
+gather / scatter that feeds the MAM fully-connected kernel with convolution windows
+(mamtorch/kernel/backup/mamconv1d_forward.txt, mamconv2d_forward.txt)."""
+import torch
+from torch import Tensor
+
+__all__ = ["blend", "im2col", "col2im"]
+
+K = torch.ops.mamtorch_kernel_v4
+
+
+def blend(mam: Tensor, mac: Tensor, bias, alpha: float, beta: float) -> Tensor:
+    """(alpha * mam + beta * mac) + bias in the reference's rounding order; (N, out) operands."""
+    return K.blend.default(mam, mac, bias, float(alpha), float(beta))
+
+
+def im2col(x: Tensor, k1: int, k2: int, s1: int, s2: int) -> Tensor:
+    """x (B, C, H, W) -> (B * L1 * L2, k2 * k1 * C) windows, column (j2 * k1 + j1) * C + c."""
+    return K.im2col.default(x, k1, k2, s1, s2)
+
+
+def col2im(cols: Tensor, shape, k1: int, k2: int, s1: int, s2: int) -> Tensor:
+    """Adjoint of :func:`im2col`: (B * L1 * L2, k2 * k1 * C) -> (B, C, H, W), overlapping windows add up."""
+    B, C, H, W = shape
+    return K.col2im.default(cols, B, C, H, W, k1, k2, s1, s2)
+
+
+@torch.library.register_fake("mamtorch_kernel_v4::blend")
+def _(mam, mac, bias, alpha, beta):
+    torch._check(mam.dim() == 2 and mam.shape == mac.shape)
+    torch._check(mam.dtype == torch.float and mac.dtype == torch.float)
+    return torch.empty(mam.shape, dtype=torch.float, device=mam.device)
+
+
+def _blend_setup(ctx, inputs, output):
+    _, _, _, alpha, beta = inputs
+    ctx.alpha, ctx.beta = alpha, beta
+
+
+def _blend_backward(ctx, grad):
+    g_mam = grad * ctx.alpha if ctx.needs_input_grad[0] else None
+    g_mac = grad * ctx.beta if ctx.needs_input_grad[1] else None
+    g_bias = grad.sum(dim=0) if ctx.needs_input_grad[2] else None
+    return g_mam, g_mac, g_bias, None, None
+
+
+torch.library.register_autograd("mamtorch_kernel_v4::blend", _blend_backward, setup_context=_blend_setup)
+
+
+def _out_positions(H, W, k1, k2, s1, s2):
+    return (H - k1) // s1 + 1, (W - k2) // s2 + 1
+
+
+@torch.library.register_fake("mamtorch_kernel_v4::im2col")
+def _(x, k1, k2, s1, s2):
+    torch._check(x.dim() == 4 and x.dtype == torch.float)
+    B, C, H, W = x.shape
+    L1, L2 = _out_positions(H, W, k1, k2, s1, s2)
+    return torch.empty((B * L1 * L2, k2 * k1 * C), dtype=torch.float, device=x.device)
+
+
+@torch.library.register_fake("mamtorch_kernel_v4::col2im")
+def _(cols, B, C, H, W, k1, k2, s1, s2):
+    torch._check(cols.dim() == 2 and cols.dtype == torch.float)
+    return torch.empty((B, C, H, W), dtype=torch.float, device=cols.device)
+
+
+def _im2col_setup(ctx, inputs, output):
+    x, k1, k2, s1, s2 = inputs
+    ctx.geom = (tuple(x.shape), k1, k2, s1, s2)
+
+
+def _im2col_backward(ctx, grad):
+    shape, k1, k2, s1, s2 = ctx.geom
+    return K.col2im.default(grad.contiguous(), *shape, k1, k2, s1, s2), None, None, None, None
+
+
+torch.library.register_autograd("mamtorch_kernel_v4::im2col", _im2col_backward, setup_context=_im2col_setup)
+
+
+def _col2im_setup(ctx, inputs, output):
+    ctx.geom = inputs[5:]
+
+
+def _col2im_backward(ctx, grad):
+    k1, k2, s1, s2 = ctx.geom
+    return (K.im2col.default(grad.contiguous(), k1, k2, s1, s2),) + (None,) * 8
+
+
+torch.library.register_autograd("mamtorch_kernel_v4::col2im", _col2im_backward, setup_context=_col2im_setup)

@@ -6,10 +6,11 @@ Stands in for the two advanced-index updates of FullyConnected.update_selection_
 import torch
 from torch import Tensor
 
-__all__ = ["selection_count", "COUNT_REFERENCE", "COUNT_HITS"]
+__all__ = ["selection_count", "COUNT_REFERENCE", "COUNT_HITS", "COUNT_FLAGS"]
 
 COUNT_REFERENCE = 0  # literal module behaviour: de-duplicated per call, both into max_count
 COUNT_HITS = 1       # true hit counts, argmax into max_count and argmin into min_count
+COUNT_FLAGS = 2      # de-duplicated per call like COUNT_REFERENCE, but max and min into their own counters
 
 K = torch.ops.mamtorch_kernel_v4
 

@@ -172,7 +172,7 @@ class FullyConnected(Module):
         w = self._dropped_weight()
         # the bias rides along in the kernel when nothing is added between MAM and bias (no MAC
         # blend, no sum over splits), which keeps the reference's rounding order (max+min)+bias
-        fuse_bias = self.bias is not None and self.beta == 0 and self.alpha == 1.0 and self.splits == 1
+        fuse_bias = self.bias is not None and self.beta == 0 and self.splits == 1
         fused = self.bias if fuse_bias else None
 
         if self.splits > 1:
@@ -192,10 +192,10 @@ class FullyConnected(Module):
                 C_flat = self._mam_noargs(input_flat, w, fused)
 
         if self.beta > 0:
+            # alpha * MAM + beta * MAC + bias as one kernel, in the reference's rounding order
             mac_weight = self.weight.detach() if self.train_mam_only else self.weight
-            C_flat = self.alpha * C_flat + self.beta * F.linear(input_flat, mac_weight)
-
-        if self.bias is not None and not fuse_bias:
+            C_flat = K.v4.blend(C_flat, F.linear(input_flat, mac_weight), self.bias, self.alpha, self.beta)
+        elif self.bias is not None and not fuse_bias:
             C_flat = C_flat + self.bias.view(1, -1)
 
         C = C_flat.view(input.shape[:-1] + (self.weight.size(0),))

@@ -146,3 +146,34 @@ def csr_spmm(crow, col, val, b):
     R = crow.shape[0] - 1
     row = np.repeat(np.arange(R, dtype=np.int64), np.diff(crow))
     return coo_spmm(row, col, val, b, R)
+
+
+def conv_windows(x, k1, k2, s1, s2):
+    """x (B, C, H, W) -> the (B * L1 * L2, k2 * k1 * C) matrix of windows, column
+    q = (j2 * k1 + j1) * C + c, built by plain numpy slicing (one slice per window position): the operand on
+    which forward() gives the MAM convolution of brute.conv_forward at sizes the pure-Python loops cannot
+    reach.  Pinned against brute.conv_forward in tests/test_oracle.py."""
+    x = np.asarray(x, dtype=np.float32)
+    B, C, H, W = x.shape
+    L1, L2 = (H - k1) // s1 + 1, (W - k2) // s2 + 1
+    cols = np.empty((B, L1, L2, k2, k1, C), dtype=np.float32)
+    for j2 in range(k2):
+        for j1 in range(k1):
+            # x[b, c, l1 * s1 + j1, l2 * s2 + j2] for all (b, c, l1, l2)
+            win = x[:, :, j1:j1 + (L1 - 1) * s1 + 1:s1, j2:j2 + (L2 - 1) * s2 + 1:s2]
+            cols[:, :, :, j2, j1, :] = win.transpose(0, 2, 3, 1)
+    return cols.reshape(B * L1 * L2, k2 * k1 * C)
+
+
+def conv_forward(x, w, stride=(1, 1), bias=None):
+    """MAM convolution through conv_windows + forward(): y, argmax, argmin of shape (B, F, L1, L2)."""
+    x = np.asarray(x, dtype=np.float32)
+    w = np.asarray(w, dtype=np.float32)
+    B, C, H, W = x.shape
+    Fo, _, k1, k2 = w.shape
+    s1, s2 = stride
+    L1, L2 = (H - k1) // s1 + 1, (W - k2) // s2 + 1
+    wm = np.ascontiguousarray(w.transpose(0, 3, 2, 1).reshape(Fo, k2 * k1 * C))
+    c, amax, amin = forward(conv_windows(x, k1, k2, s1, s2), wm, W_MK, bias)
+    shape = (B, L1, L2, Fo)
+    return tuple(np.ascontiguousarray(t.reshape(shape).transpose(0, 3, 1, 2)) for t in (c, amax, amin))

@@ -67,3 +67,68 @@ def selection_count(argmax, argmin, max_count, min_count, mode=0):
         for (m, k) in cells:
             mc[m, k] += 1
     return mc, nc
+
+
+def conv_forward(x, w, stride=(1, 1), bias=None):
+    """MAM convolution by its scalar definition.  x (B, C, H, W), w (F, C, k1, k2), no padding ->
+    y, argmax, argmin of shape (B, F, L1, L2).  Products are scanned in ascending
+    q = (j2 * k1 + j1) * C + c (window column outermost, then window row, channel innermost) with strict
+    comparisons, the order in which the reference's kernels walk a window
+    (mamtorch/kernel/backup/mamconv1d_forward.txt:74-139: blocks of k over position * C + channel;
+    index decoding in mamtorch/nn/backup/mamconv2d.txt:97-103).  A 1-D convolution is H = k1 = 1."""
+    x = np.asarray(x, f32)
+    w = np.asarray(w, f32)
+    B, C, H, W = x.shape
+    Fo, _, k1, k2 = w.shape
+    s1, s2 = stride
+    L1, L2 = (H - k1) // s1 + 1, (W - k2) // s2 + 1
+    y = np.zeros((B, Fo, L1, L2), f32)
+    amax = np.zeros((B, Fo, L1, L2), np.int32)
+    amin = np.zeros((B, Fo, L1, L2), np.int32)
+    for b in range(B):
+        for f in range(Fo):
+            for l1 in range(L1):
+                for l2 in range(L2):
+                    hi = lo = None
+                    ih = il = 0
+                    for j2 in range(k2):
+                        for j1 in range(k1):
+                            for c in range(C):
+                                q = (j2 * k1 + j1) * C + c
+                                p = f32(x[b, c, l1 * s1 + j1, l2 * s2 + j2]) * f32(w[f, c, j1, j2])
+                                if hi is None or p > hi:
+                                    hi, ih = p, q
+                                if lo is None or p < lo:
+                                    lo, il = p, q
+                    s = f32(hi + lo)
+                    if bias is not None:
+                        s = f32(s + f32(bias[f]))
+                    y[b, f, l1, l2], amax[b, f, l1, l2], amin[b, f, l1, l2] = s, ih, il
+    return y, amax, amin
+
+
+def conv_backward(x, w, grad, argmax, argmin, stride=(1, 1)):
+    """-> x_grad like x, w_grad like w (fp64 accumulation of fp32 terms): the gradient goes to the two
+    selected (input, weight) pairs of every output position, twice when they coincide
+    (mamtorch/kernel/backup/mamconv1d_backward.txt)."""
+    x = np.asarray(x, f32)
+    w = np.asarray(w, f32)
+    grad = np.asarray(grad, f32)
+    B, C, H, W = x.shape
+    Fo, _, k1, k2 = w.shape
+    s1, s2 = stride
+    xg = np.zeros(x.shape, np.float64)
+    wg = np.zeros(w.shape, np.float64)
+    _, _, L1, L2 = grad.shape
+    for b in range(B):
+        for f in range(Fo):
+            for l1 in range(L1):
+                for l2 in range(L2):
+                    g = grad[b, f, l1, l2]
+                    for q in (int(argmax[b, f, l1, l2]), int(argmin[b, f, l1, l2])):
+                        c, pos = q % C, q // C
+                        j1, j2 = pos % k1, pos // k1
+                        h, ww = l1 * s1 + j1, l2 * s2 + j2
+                        xg[b, c, h, ww] += float(f32(w[f, c, j1, j2]) * g)
+                        wg[f, c, j1, j2] += float(f32(x[b, c, h, ww]) * g)
+    return xg.astype(f32), wg.astype(f32)

@@ -315,3 +315,54 @@ def test_prune_oracle_against_the_literal_torch_rule(p):
         np.testing.assert_array_equal(col[kept_nonzero], csr.col_indices().numpy())
         np.testing.assert_array_equal(val[kept_nonzero], csr.values().numpy())
         assert crow[-1] == len(col) and abs(len(col) / w.numel() - (1 - p)) < 0.02
+
+
+def test_conv_oracle_known_answers_and_cross_checks():
+    """The MAM convolution of the reference's retired kernels: hand-derived known answers
+    (tests/golden/kat_conv.json), the numpy window builder + C oracle against the pure-Python scalar
+    loops, the window matrix against torch's own unfold (other column order, permuted here), and the
+    backward against autograd of the gather formulation."""
+    import json
+    import os
+
+    import torch
+    import torch.nn.functional as F
+    from oracle import brute
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    for kat in json.load(open(os.path.join(here, "golden", "kat_conv.json"))):
+        x = np.array(kat["x"], np.float32)[:, :, None, :]
+        w = np.array(kat["w"], np.float32)[:, :, None, :]
+        for fn in (brute.conv_forward, oracle.conv_forward):
+            y, amax, amin = fn(x, w, (1, kat["stride"]))
+            assert y[:, :, 0].tolist() == kat["y"], kat["name"]
+            assert amax[:, :, 0].tolist() == kat["argmax"] and amin[:, :, 0].tolist() == kat["argmin"], kat["name"]
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 3, 6, 7)).astype(np.float32)
+    w = rng.standard_normal((4, 3, 2, 3)).astype(np.float32)
+    bias = rng.standard_normal(4).astype(np.float32)
+    for stride in ((1, 1), (2, 1), (1, 3)):
+        a = brute.conv_forward(x, w, stride, bias)
+        b = oracle.conv_forward(x, w, stride, bias)
+        assert all(np.array_equal(u.view(np.int32), v.view(np.int32)) for u, v in zip(a, b))
+        # torch's unfold orders columns (c, j1, j2); ours is (j2, j1, c)
+        cols = oracle.conv_windows(x, 2, 3, *stride)
+        unf = F.unfold(torch.tensor(x), (2, 3), stride=stride)                     # (B, C*k1*k2, L)
+        unf = unf.view(2, 3, 2, 3, -1).permute(0, 4, 3, 2, 1).reshape(cols.shape)   # (B, L, j2, j1, c)
+        assert np.array_equal(cols, unf.numpy())
+        # backward: autograd of y = p[argmax] + p[argmin] over the window matrix
+        grad = rng.standard_normal(a[0].shape).astype(np.float32)
+        xg, wg = brute.conv_backward(x, w, grad, a[1], a[2], stride)
+        xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+        wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+        u = F.unfold(xt, (2, 3), stride=stride).view(2, 3, 2, 3, -1).permute(0, 4, 3, 2, 1).reshape(cols.shape[0], -1)
+        wm = wt.permute(0, 3, 2, 1).reshape(4, -1)
+        prods = u[:, None, :] * wm[None, :, :]                                      # (rows, F, q)
+        L = a[1].shape[2] * a[1].shape[3]
+        i1 = torch.tensor(a[1]).permute(0, 2, 3, 1).reshape(-1, 4, 1).long()
+        i2 = torch.tensor(a[2]).permute(0, 2, 3, 1).reshape(-1, 4, 1).long()
+        yy = prods.gather(2, i1) + prods.gather(2, i2)
+        gflat = torch.tensor(grad, dtype=torch.float64).permute(0, 2, 3, 1).reshape(-1, 4, 1)
+        (yy * gflat).sum().backward()
+        assert np.allclose(xg, xt.grad.numpy(), rtol=1e-5, atol=1e-6) and np.allclose(wg, wt.grad.numpy(), rtol=1e-5, atol=1e-6)
+        assert L > 0
