@@ -159,6 +159,27 @@ int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, in
                     const float *x_sel, float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, void *stream);
 
 /*
+ * The module's `splits` in one call each way (mamtorch/nn/v4/fullyconnected.py:163-176 runs one operator
+ * per slice of the input and adds the slices' outputs with ATen).  K is cut into consecutive ranges of
+ * `range_len` inputs, the last one shorter; every range is a MAM neuron of its own:
+ *   c[n,m] = ((v_0 + v_1) + v_2 ...) (+ bias[m]),  v_r = max_{k in range r} x*w + min_{k in range r} x*w,
+ * added in ascending range order and then the bias, which is the rounding order of the reference's
+ * `C_flat += ...` statements.  argmax / argmin (both or neither; NULL = values only, the eval path):
+ * [ranges][N][M] int32, plane r holding the lowest ABSOLUTE k of range r attaining its extreme (the
+ * reference's per-slice operators return k relative to the slice).  `workspace`:
+ * mam_fc_forward_ranges_workspace() bytes (0 when range_len >= K, which is mam_fc_forward).
+ *   mam_fc_backward_ranges: the gradient of that c: every range routes grad[n,m] to its own two
+ * selected positions.  x_grad (N,K), w_grad (shape and layout of w), either may be NULL.
+ */
+size_t mam_fc_forward_ranges_workspace(int64_t N, int64_t K, int64_t M, int64_t range_len, int with_indices);
+int mam_fc_forward_ranges(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                          const float *bias, float *c, int32_t *argmax, int32_t *argmin, int64_t N, int64_t K,
+                          int64_t M, int64_t range_len, void *workspace, size_t workspace_bytes, void *stream);
+int mam_fc_backward_ranges(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                           const float *grad, const int32_t *argmax, const int32_t *argmin, float *x_grad,
+                           float *w_grad, int64_t N, int64_t K, int64_t M, int64_t range_len, void *stream);
+
+/*
  * Selection-count accumulation for pruning: adds this batch's picks into (M,K) int32 counters
  * in place.  Replaces FullyConnected.update_selection_count
  * (mamtorch/nn/v4/fullyconnected.py:114-129).  min_count may be NULL in MAM_COUNT_REFERENCE mode.

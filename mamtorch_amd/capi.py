@@ -30,6 +30,7 @@ EXPORTS = (
     "mam_fc_forward_workspace", "mam_fc_forward",
     "mam_fc_forward_values_workspace", "mam_fc_forward_values",
     "mam_fc_backward", "mam_selection_count",
+    "mam_fc_forward_ranges_workspace", "mam_fc_forward_ranges", "mam_fc_backward_ranges",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward", "mam_csr_validate",
     "mam_csr_spmm", "mam_coo_spmm",
     "mam_blend", "mam_im2col", "mam_col2im",
@@ -68,6 +69,12 @@ def lib():
                                             _ptr, _size, _ptr]
         l.mam_fc_backward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                       _i64, _i64, _i64, _ptr]
+        l.mam_fc_forward_ranges_workspace.restype = _size
+        l.mam_fc_forward_ranges_workspace.argtypes = [_i64, _i64, _i64, _i64, _int]
+        l.mam_fc_forward_ranges.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64,
+                                            _i64, _ptr, _size, _ptr]
+        l.mam_fc_backward_ranges.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
+                                             _i64, _i64, _ptr]
         l.mam_selection_count.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr]
         l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                          _i64, _i64, _i64, _i64, _ptr, _size, _ptr]
@@ -172,6 +179,34 @@ def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=Tru
     with torch.cuda.device(x.device):
         _check(l.mam_fc_backward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(grad), _p(argmax), _p(argmin),
                                  _p(w_sel), _p(x_sel), _p(xg), _p(wg), N, K, M, _stream(x)))
+    return xg, wg
+
+
+def fc_forward_ranges(x, w, range_len, layout=W_KM, bias=None, with_indices=True):
+    """-> (c, argmax, argmin) with argmax / argmin of shape (ranges, N, M) holding absolute k (None, None
+    when with_indices is false): the module's `splits` as one call."""
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    ranges = max(1, -(-K // range_len))
+    c = torch.empty((N, M), dtype=torch.float32, device=x.device)
+    amax = torch.empty((ranges, N, M), dtype=torch.int32, device=x.device) if with_indices else None
+    amin = torch.empty((ranges, N, M), dtype=torch.int32, device=x.device) if with_indices else None
+    need = l.mam_fc_forward_ranges_workspace(N, K, M, range_len, int(with_indices))
+    ws = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        _check(l.mam_fc_forward_ranges(_p(x), _ld(x), _p(w), _ld(w), layout, _p(bias), _p(c), _p(amax), _p(amin),
+                                       N, K, M, range_len, _p(ws), need, _stream(x)))
+    return c, amax, amin
+
+
+def fc_backward_ranges(x, w, grad, argmax, argmin, range_len, layout=W_KM, want_x=True, want_w=True):
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    xg = torch.empty((N, K), dtype=torch.float32, device=x.device) if want_x else None
+    wg = torch.empty(tuple(w.shape), dtype=torch.float32, device=x.device) if want_w else None
+    with torch.cuda.device(x.device):
+        _check(l.mam_fc_backward_ranges(_p(x), _ld(x), _p(w), _ld(w), layout, _p(grad), _p(argmax), _p(argmin),
+                                        _p(xg), _p(wg), N, K, M, range_len, _stream(x)))
     return xg, wg
 
 

@@ -53,18 +53,22 @@ template <int LAYOUT>
 __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
     const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int K, int M, int kc)
+    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int K, int M, int kc, int planes)
 {
+    // planes > 1 (the module's `splits`): argmax / argmin are [plane][N*M] arrays of absolute k, one pair
+    // per K range, w_sel (if any) [plane][2][N*M]; every plane scatters the same grad
     extern __shared__ float hist[];
     const int n = blockIdx.x;
     const int tid = threadIdx.x;
     const float *g_row = grad + (int64_t)n * M;
-    const int32_t *amax_row = argmax + (int64_t)n * M;
-    const int32_t *amin_row = argmin + (int64_t)n * M;
     for (int k0 = 0; k0 < K; k0 += kc) {
         const int kn = (K - k0) < kc ? (K - k0) : kc;
         for (int i = tid; i < kn; i += NT_X) hist[i] = 0.0f;
         __syncthreads();
+        for (int pl = 0; pl < planes; ++pl) {
+        const int32_t *amax_row = argmax + pl * nm + (int64_t)n * M;
+        const int32_t *amin_row = argmin + pl * nm + (int64_t)n * M;
+        const float *w_sel_pl = w_sel ? w_sel + pl * 2 * nm : nullptr;
         // four outputs per thread and trip: all index loads, then all weight gathers, then the
         // LDS adds, so that the gather latencies overlap instead of adding up
         for (int mb = tid; mb < M; mb += 4 * NT_X) {
@@ -82,10 +86,10 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
             for (int u = 0; u < 4; ++u) {
                 const int m = mb + u * NT_X;
                 // the forward can hand over the selected weights; otherwise gather them
-                if (w_sel) {
+                if (w_sel_pl) {
                     const bool ok = m < M;
-                    wv1[u] = ok ? w_sel[(int64_t)n * M + m] : 0.0f;
-                    wv2[u] = ok ? w_sel[nm + (int64_t)n * M + m] : 0.0f;
+                    wv1[u] = ok ? w_sel_pl[(int64_t)n * M + m] : 0.0f;
+                    wv2[u] = ok ? w_sel_pl[nm + (int64_t)n * M + m] : 0.0f;
                 } else {
                     wv1[u] = (unsigned)a1[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a1[u] + k0, m) : 0.0f;
                     wv2[u] = (unsigned)a2[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a2[u] + k0, m) : 0.0f;
@@ -96,6 +100,7 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
                 if ((unsigned)a1[u] < (unsigned)kn) lds_add(&hist[a1[u]], wv1[u] * g[u]);
                 if ((unsigned)a2[u] < (unsigned)kn) lds_add(&hist[a2[u]], wv2[u] * g[u]);
             }
+        }
         }
         __syncthreads();
         float *dst = x_grad + (int64_t)n * K + k0;
@@ -114,7 +119,8 @@ template <int LAYOUT>
 __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
     const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int N, int K, int M, int log2r)
+    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int N, int K, int M, int log2r,
+    int planes)
 {
     extern __shared__ float hist[];   // [R][K]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -129,15 +135,20 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
 
     float4 g = make_float4(0.f, 0.f, 0.f, 0.f), s1 = g, s2 = g;
     int4 i1, i2;
+    float *row = hist + r * K;
+    const int trips = (M + m_step - 1) / m_step;     // the same for every thread: lanes past M hold no item
+    for (int pl = 0; pl < planes; ++pl) {            // one (argmax, argmin) pair per K range
+    const int32_t *amax_pl = argmax + pl * nm, *amin_pl = argmin + pl * nm;
+    const float *w_sel_pl = w_sel ? w_sel + pl * 2 * nm : nullptr;
     auto load = [&](int m) {
         if (row_ok && m < M) {
             const int64_t o = (int64_t)n * M + m;
             g = *reinterpret_cast<const float4 *>(grad + o);
-            i1 = *reinterpret_cast<const int4 *>(argmax + o);
-            i2 = *reinterpret_cast<const int4 *>(argmin + o);
-            if (w_sel) {
-                s1 = *reinterpret_cast<const float4 *>(w_sel + o);
-                s2 = *reinterpret_cast<const float4 *>(w_sel + nm + o);
+            i1 = *reinterpret_cast<const int4 *>(amax_pl + o);
+            i2 = *reinterpret_cast<const int4 *>(amin_pl + o);
+            if (w_sel_pl) {
+                s1 = *reinterpret_cast<const float4 *>(w_sel_pl + o);
+                s2 = *reinterpret_cast<const float4 *>(w_sel_pl + nm + o);
             }
         } else {
             i1 = make_int4(-1, -1, -1, -1);
@@ -146,8 +157,6 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
     };
     int m = (wave * lpr + j) * 4;
     load(m);
-    float *row = hist + r * K;
-    const int trips = (M + m_step - 1) / m_step;     // the same for every thread: lanes past M hold no item
     for (int t = 0; t < trips; ++t) {
         const float4 cg = g, c1 = s1, c2 = s2;
         const int4 a1 = i1, a2 = i2;
@@ -169,6 +178,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
             if ((unsigned)k1[u] < (unsigned)K) lds_add_sparse(&row[k1[u]], w1[u] * gv[u]);
             if ((unsigned)k2[u] < (unsigned)K) lds_add_sparse(&row[k2[u]], w2[u] * gv[u]);
         }
+    }
     }
     __syncthreads();
     const int rows = (N - blockIdx.x * R) < R ? (N - blockIdx.x * R) : R;
@@ -263,7 +273,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
     const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
-    int kc, int vec_out, int mtiles, int tiles_per_wg, int rows_per_split)
+    int kc, int vec_out, int mtiles, int tiles_per_wg, int rows_per_split, int planes, int range_len)
 {
     extern __shared__ float hist[];
     const int tid = threadIdx.x;
@@ -273,13 +283,23 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
     const int n_begin = blockIdx.z * rows_per_split;
     const int n_rows = (N - n_begin) < rows_per_split ? (N - n_begin) : rows_per_split;
     const bool accumulate = gridDim.z > 1;
-    const int64_t items = (int64_t)n_rows * qpr;
     const int k0 = blockIdx.y * kc;
     const int kn = (K - k0) < kc ? (K - k0) : kc;
+    // planes > 1 (the module's `splits`): one (argmax, argmin) pair of absolute k per K range of
+    // `range_len`, [plane][N*M]; a slab takes the planes whose ranges meet its k chunk
+    const int pl_lo = planes > 1 ? k0 / range_len : 0;
+    int pl_hi = planes > 1 ? (k0 + kn - 1) / range_len : 0;
+    pl_hi = pl_hi < planes - 1 ? pl_hi : planes - 1;
+    const int npl = pl_hi - pl_lo + 1;
+    const int64_t per_plane = (int64_t)n_rows * qpr;
+    const int64_t items = per_plane * npl;
     const int first = xcd_remap(blockIdx.x, gridDim.x) * tiles_per_wg;
 
-    // this thread's first item of a slab: row n_first, neurons m0 + r_first .. +3
-    const int n_first = n_begin + tid / qpr, r_first = (tid % qpr) * 4;
+    // this thread's first item of a slab: plane pl_lo + pf, row n_first, neurons m0 + r_first .. +3
+    const int pf = npl > 1 ? (int)(tid / per_plane) : 0;
+    const int rem_first = npl > 1 ? (int)(tid - pf * per_plane) : tid;
+    const int n_first = n_begin + rem_first / qpr, r_first = (rem_first % qpr) * 4;
+    const int64_t po_first = (int64_t)(pl_lo + pf) * nm;
     float4 g = make_float4(0.f, 0.f, 0.f, 0.f);
     float4 s1 = g, s2 = g;      // selected inputs handed over by the forward, if any
     int4 i1 = make_int4(-1, -1, -1, -1), i2 = make_int4(-1, -1, -1, -1);
@@ -289,11 +309,11 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
         if (have) {
             const int64_t o = (int64_t)n_first * M + m0 + r_first;
             g = *reinterpret_cast<const float4 *>(grad + o);
-            i1 = *reinterpret_cast<const int4 *>(argmax + o);
-            i2 = *reinterpret_cast<const int4 *>(argmin + o);
+            i1 = *reinterpret_cast<const int4 *>(argmax + po_first + o);
+            i2 = *reinterpret_cast<const int4 *>(argmin + po_first + o);
             if (x_sel) {
-                s1 = *reinterpret_cast<const float4 *>(x_sel + o);
-                s2 = *reinterpret_cast<const float4 *>(x_sel + nm + o);
+                s1 = *reinterpret_cast<const float4 *>(x_sel + 2 * po_first + o);
+                s2 = *reinterpret_cast<const float4 *>(x_sel + 2 * po_first + nm + o);
             }
         }
     };
@@ -311,16 +331,19 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
         __syncthreads();
         if (have) scatter_quad<LAYOUT>(hist, g, i1, i2, x1, x2, r_first, k0, kn, kc, log2r);
         for (int64_t it = tid + NT_W; it < items; it += NT_W) {
-            const int n = n_begin + (int)(it / qpr), r0 = (int)(it % qpr) * 4;
+            const int pl = npl > 1 ? (int)(it / per_plane) : 0;
+            const int64_t rem = npl > 1 ? it - pl * per_plane : it;
+            const int n = n_begin + (int)(rem / qpr), r0 = (int)(rem % qpr) * 4;
             if (m0 + r0 >= M) continue;
             const int64_t o = (int64_t)n * M + m0 + r0;
+            const int64_t po = (int64_t)(pl_lo + pl) * nm;
             const float4 gg = *reinterpret_cast<const float4 *>(grad + o);
-            const int4 j1 = *reinterpret_cast<const int4 *>(argmax + o);
-            const int4 j2 = *reinterpret_cast<const int4 *>(argmin + o);
+            const int4 j1 = *reinterpret_cast<const int4 *>(argmax + po + o);
+            const int4 j2 = *reinterpret_cast<const int4 *>(argmin + po + o);
             float y1[4], y2[4];
             if (x_sel) {
-                const float4 t1 = *reinterpret_cast<const float4 *>(x_sel + o);
-                const float4 t2 = *reinterpret_cast<const float4 *>(x_sel + nm + o);
+                const float4 t1 = *reinterpret_cast<const float4 *>(x_sel + 2 * po + o);
+                const float4 t2 = *reinterpret_cast<const float4 *>(x_sel + 2 * po + nm + o);
                 y1[0] = t1.x; y1[1] = t1.y; y1[2] = t1.z; y1[3] = t1.w;
                 y2[0] = t2.x; y2[1] = t2.y; y2[2] = t2.z; y2[3] = t2.w;
             } else {
@@ -341,7 +364,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
     const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
-    int kc, int vec_out)
+    int kc, int vec_out, int planes, int range_len)
 {
     extern __shared__ float hist[];
     const int tid = threadIdx.x;
@@ -356,19 +379,27 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
         *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
     const int64_t pairs = (int64_t)N << log2r;
-    for (int64_t pi = tid; pi < pairs; pi += NT_W) {
-        const int n = (int)(pi >> log2r), r = (int)(pi & (R - 1));
-        if (r >= rn) continue;
-        const int64_t o = (int64_t)n * M + m0 + r;
-        const float g = grad[o];
-        const int a1 = argmax[o] - k0, a2 = argmin[o] - k0;
-        const float *xr = x + (int64_t)n * ldx + k0;
-        if ((unsigned)a1 < (unsigned)kn)
-            lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r],
-                           (x_sel ? x_sel[o] : xr[a1]) * g);
-        if ((unsigned)a2 < (unsigned)kn)
-            lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r],
-                           (x_sel ? x_sel[nm + o] : xr[a2]) * g);
+    // one (argmax, argmin) pair of absolute k per K range; only the planes whose ranges meet this k chunk
+    const int pl_lo = planes > 1 ? k0 / range_len : 0;
+    int pl_hi = planes > 1 ? (k0 + kn - 1) / range_len : 0;
+    pl_hi = pl_hi < planes - 1 ? pl_hi : planes - 1;
+    for (int pl = pl_lo; pl <= pl_hi; ++pl) {
+        const int32_t *amax_pl = argmax + pl * nm, *amin_pl = argmin + pl * nm;
+        const float *x_sel_pl = x_sel ? x_sel + pl * 2 * nm : nullptr;
+        for (int64_t pi = tid; pi < pairs; pi += NT_W) {
+            const int n = (int)(pi >> log2r), r = (int)(pi & (R - 1));
+            if (r >= rn) continue;
+            const int64_t o = (int64_t)n * M + m0 + r;
+            const float g = grad[o];
+            const int a1 = amax_pl[o] - k0, a2 = amin_pl[o] - k0;
+            const float *xr = x + (int64_t)n * ldx + k0;
+            if ((unsigned)a1 < (unsigned)kn)
+                lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a1 : (a1 << log2r) + r],
+                               (x_sel_pl ? x_sel_pl[o] : xr[a1]) * g);
+            if ((unsigned)a2 < (unsigned)kn)
+                lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a2 : (a2 << log2r) + r],
+                               (x_sel_pl ? x_sel_pl[nm + o] : xr[a2]) * g);
+        }
     }
     __syncthreads();
     store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, false);
@@ -402,9 +433,11 @@ static DeviceHookRegistration g_registration(setup_device);
 template <int LAYOUT>
 static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ldw, const float *grad,
                          const int32_t *argmax, const int32_t *argmin, const float *w_sel, const float *x_sel,
-                         float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
+                         float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, hipStream_t st,
+                         int planes = 1, int range_len = 0)
 {
     int rc = MAM_OK;
+    if (planes <= 1) range_len = (int)K;
     const int dev = ensure_device();
     if (dev < 0) return dev;
     const int lds_cap = g_lds_floats[dev];
@@ -419,14 +452,14 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         const int R = 1 << log2r;
         hipLaunchKernelGGL((mam_bwd_x_rows_kernel<LAYOUT>), dim3((unsigned)ceil_div(N, R)), dim3(NT_W),
                            (size_t)R * K * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M, x_grad,
-                           (int)N, (int)K, (int)M, log2r);
+                           (int)N, (int)K, (int)M, log2r, planes);
         rc = check_launch("mam_bwd_x_rows_kernel");
         if (rc != MAM_OK) return rc;
     } else if (x_grad) {
         const int kc = (int)(K < lds_cap ? K : lds_cap);
         hipLaunchKernelGGL((mam_bwd_x_kernel<LAYOUT>), dim3((unsigned)N), dim3(NT_X),
                            (size_t)kc * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M,
-                           x_grad, (int)K, (int)M, kc);
+                           x_grad, (int)K, (int)M, kc, planes);
         rc = check_launch("mam_bwd_x_kernel");
         if (rc != MAM_OK) return rc;
     }
@@ -477,11 +510,12 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
                                dim3((unsigned)ceil_div(mtiles, tpw), (unsigned)ktiles, (unsigned)shares), dim3(NT_W),
                                (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax, argmin, x_sel, N * M,
                                w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out, (int)mtiles, tpw,
-                               (int)rows_per_share);
+                               (int)rows_per_share, planes, range_len);
         } else {
             hipLaunchKernelGGL((mam_bwd_w_kernel<LAYOUT>), dim3((unsigned)mtiles, (unsigned)ktiles),
                                dim3(NT_W), (size_t)R * kc * sizeof(float), st, x, ldx, grad, argmax,
-                               argmin, x_sel, N * M, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out);
+                               argmin, x_sel, N * M, w_grad, (int)N, (int)K, (int)M, log2r, kc, vec_out, planes,
+                               range_len);
         }
         rc = check_launch("mam_bwd_w_kernel");
     }
@@ -497,17 +531,17 @@ int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t
     const int kc = (int)(K < g_lds_floats[dev] ? K : g_lds_floats[dev]);
     hipLaunchKernelGGL((mam_bwd_x_kernel<MAM_W_MK>), dim3((unsigned)N), dim3(NT_X), (size_t)kc * sizeof(float),
                        st, (const float *)nullptr, (int64_t)0, grad, argmax, argmin, w_sel, N * M, x_grad, (int)K,
-                       (int)M, kc);
+                       (int)M, kc, 1);
     return check_launch("mam_bwd_x_kernel");
 }
 
 }  // namespace bwd
 }  // namespace mam
 
-extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
-                               const float *grad, const int32_t *argmax, const int32_t *argmin,
-                               const float *w_sel, const float *x_sel, float *x_grad, float *w_grad,
-                               int64_t N, int64_t K, int64_t M, void *stream)
+static int backward_impl(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                         const float *grad, const int32_t *argmax, const int32_t *argmin,
+                         const float *w_sel, const float *x_sel, float *x_grad, float *w_grad,
+                         int64_t N, int64_t K, int64_t M, int planes, int range_len, void *stream)
 {
     using namespace mam;
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
@@ -528,8 +562,10 @@ extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int6
         return fail(MAM_ERR_INVALID_ARGUMENT, "leading dimension smaller than the row length");
     auto launch = [&](float *xg, float *wg, hipStream_t on) {
         if (w_layout == MAM_W_MK)
-            return bwd::launch_layout<MAM_W_MK>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, xg, wg, N, K, M, on);
-        return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, xg, wg, N, K, M, on);
+            return bwd::launch_layout<MAM_W_MK>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, xg, wg, N, K, M, on,
+                                                planes, range_len);
+        return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, xg, wg, N, K, M, on,
+                                            planes, range_len);
     };
     // x_grad is bound by LDS atomics and w_grad by memory traffic, and neither depends on the other
     if (x_grad && w_grad) {
@@ -543,4 +579,25 @@ extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int6
         }
     }
     return launch(x_grad, w_grad, st);
+}
+
+extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                               const float *grad, const int32_t *argmax, const int32_t *argmin,
+                               const float *w_sel, const float *x_sel, float *x_grad, float *w_grad,
+                               int64_t N, int64_t K, int64_t M, void *stream)
+{
+    return backward_impl(x, ldx, w, ldw, w_layout, grad, argmax, argmin, w_sel, x_sel, x_grad, w_grad, N, K, M, 1, 0,
+                         stream);
+}
+
+extern "C" int mam_fc_backward_ranges(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                                      const float *grad, const int32_t *argmax, const int32_t *argmin,
+                                      float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M,
+                                      int64_t range_len, void *stream)
+{
+    if (range_len <= 0) return mam::fail(MAM_ERR_INVALID_ARGUMENT, "range_len must be positive");
+    const int64_t planes = K > 0 ? (K + range_len - 1) / range_len : 1;
+    if (planes > 65535) return mam::fail(MAM_ERR_UNSUPPORTED, "more than 65535 ranges");
+    return backward_impl(x, ldx, w, ldw, w_layout, grad, argmax, argmin, nullptr, nullptr, x_grad, w_grad, N, K, M,
+                         (int)planes, (int)(range_len < K ? range_len : K), stream);
 }

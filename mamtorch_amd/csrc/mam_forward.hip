@@ -75,18 +75,17 @@ struct Params {
 // The cost of this step is the number of cache lines each wave touches, not arithmetic, so the
 // G operands of each side are fetched with 16-byte loads when the layout allows it.
 template <int LAYOUT>
-__device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, float target,
+__device__ __forceinline__ void resolve(const Params &p, int n, int m, int kb, int klast, float target,
                                         float &val, int &idx, float &wsel, float &xsel)
 {
-    const int kb = g * G;
-    const int klast = p.K - 1;
+    // the group is k = kb .. kb + G - 1; k beyond klast (the last k of the scanned range) repeat klast
     idx = kb < klast ? kb : klast;
     val = target;
     const float *xr = p.x + (int64_t)n * p.ldx;
     wsel = load_w<LAYOUT>(p.w, p.ldw, idx, m);
     xsel = xr[idx];
     float xv[G], wv[G];
-    const bool whole = kb + G <= p.K;
+    const bool whole = kb + G <= klast + 1 && (kb & 3) == 0;
     if (whole && p.vec_x) {
 #pragma unroll
         for (int q = 0; q < G / 4; ++q) {
@@ -120,10 +119,10 @@ __device__ __forceinline__ void resolve(const Params &p, int n, int m, int g, fl
 // kept another zero's sign.  Rare (whole column of products has no positive / no negative
 // entry), so a plain scan is enough.
 template <int LAYOUT>
-__device__ __noinline__ float first_zero_product(const Params &p, int n, int m)
+__device__ __noinline__ float first_zero_product(const Params &p, int n, int m, int kbegin, int kend)
 {
     const float *xr = p.x + (int64_t)n * p.ldx;
-    for (int k = 0; k < p.K; ++k) {
+    for (int k = kbegin; k < kend; ++k) {
         const float prod = xr[k] * load_w<LAYOUT>(p.w, p.ldw, k, m);
         if (prod == 0.0f) return prod;
     }
@@ -138,11 +137,11 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
     int ih = 0, il = 0;
     float wh = 0.0f, wl = 0.0f, xh = 0.0f, xl = 0.0f;
     if (ARGS) {
-        resolve<LAYOUT>(p, n, m, gmax, vmax, hi, ih, wh, xh);
-        resolve<LAYOUT>(p, n, m, gmin, vmin, lo, il, wl, xl);
+        resolve<LAYOUT>(p, n, m, gmax * G, p.K - 1, vmax, hi, ih, wh, xh);
+        resolve<LAYOUT>(p, n, m, gmin * G, p.K - 1, vmin, lo, il, wl, xl);
     } else {
-        if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m);
-        if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m);
+        if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m, 0, p.K);
+        if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m, 0, p.K);
     }
     float s = hi + lo;
     if (p.bias) s = s + p.bias[m];
@@ -728,6 +727,49 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
 }
 
 
+// The module's `splits` (mamtorch/nn/v4/fullyconnected.py:163-176): K is cut into consecutive ranges of
+// `k_per_split` inputs (the last one shorter), every range is a MAM neuron of its own, and the layer's
+// output is the sum of the ranges' (max + min) in ascending range order, then the bias -- the rounding
+// order of the reference's `C_flat += ...` statements.  The forward kernels above run once with the ranges
+// as their K ranges and leave (max, min, group) partials per range; this kernel resolves every range's
+// extremes exactly (first index, sign of a zero) and adds them up.  argmax / argmin, when asked for, are
+// [range][N*M] planes of ABSOLUTE k.
+template <int LAYOUT, bool ARGS>
+__global__ __launch_bounds__(256) void mam_fwd_range_sum_kernel(const Params p)
+{
+    const int64_t nm = (int64_t)p.N * p.M;
+    const int patches_n = (p.N + 15) / 16;
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int pm = logical / patches_n, pn = logical - pm * patches_n;
+    const int n = pn * 16 + (threadIdx.x >> 4), m = pm * 16 + (threadIdx.x & 15);
+    if (n >= p.N || m >= p.M) return;
+    const int64_t o = (int64_t)n * p.M + m;
+    const int stride = ARGS ? 3 : 2;
+    float total = 0.0f;
+    for (int s = 0; s < p.splits; ++s) {
+        const float *base = p.part + (int64_t)s * stride * nm;
+        float hi = base[o], lo = base[nm + o];
+        const int kb = s * p.k_per_split;
+        const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
+        if (ARGS) {
+            const int pk = __float_as_int(base[2 * nm + o]);
+            int ih, il;
+            float w_unused, x_unused;
+            resolve<LAYOUT>(p, n, m, kb + (pk & 0xffff) * G, ke - 1, hi, hi, ih, w_unused, x_unused);
+            resolve<LAYOUT>(p, n, m, kb + ((pk >> 16) & 0xffff) * G, ke - 1, lo, lo, il, w_unused, x_unused);
+            p.argmax[(int64_t)s * nm + o] = ih;
+            p.argmin[(int64_t)s * nm + o] = il;
+        } else {
+            if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m, kb, ke);
+            if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m, kb, ke);
+        }
+        const float v = hi + lo;
+        total = s == 0 ? v : total + v;
+    }
+    if (p.bias) total = total + p.bias[m];
+    p.c[o] = total;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Second tiling for the (M,K) layout with whole 64-k tiles: batch rows are wave-uniform.
 //
@@ -1063,7 +1105,7 @@ struct Plan {
 
 static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                      const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel,
-                     int64_t N, int64_t K, int64_t M)
+                     int64_t N, int64_t K, int64_t M, int64_t range_len = 0)
 {
     if (N < 0 || K < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
     if (w_layout != MAM_W_KM && w_layout != MAM_W_MK)
@@ -1084,22 +1126,30 @@ static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const f
     // The wave-uniform-rows tiling takes (M,K) weights with aligned rows and whole 64-k tiles; option
     // MAM_OPT_FORWARD_TILING = MAM_FORWARD_TILING_WIDE keeps every shape on the first tiling (for
     // comparisons and tests).
+    // (range_len > 0: the caller fixes the K ranges -- the module's `splits` -- instead of the launch
+    // heuristics; the wave-uniform-rows tiling then also needs whole 64-k tiles per range)
     const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % sx::KT == 0) &&
-                        (ldw * sx::BM_MAX < (1ll << 30)) &&
+                        (range_len % sx::KT == 0) && (ldw * sx::BM_MAX < (1ll << 30)) &&
                         option(MAM_OPT_FORWARD_TILING) != MAM_FORWARD_TILING_WIDE;
     plan.use_sx = use_sx;
     const int bn = use_sx ? sx::BN : BN, bm = use_sx ? sx::BM_MAX : BM;
     p.tiles_n = (int)ceil_div(N, bn);
     p.tiles_m = (int)ceil_div(M, bm);
-    p.splits = choose_splits(N, K, M, bn, bm);
-    const int kt = use_sx ? sx::KT : KT;
-    p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), kt) * kt);
+    if (range_len > 0) {
+        p.k_per_split = (int)(range_len < K ? range_len : K);
+    } else {
+        p.splits = choose_splits(N, K, M, bn, bm);
+        const int kt = use_sx ? sx::KT : KT;
+        p.k_per_split = (int)(ceil_div(ceil_div(K, p.splits), kt) * kt);
+    }
     p.splits = (int)ceil_div(K, p.k_per_split);
     p.part = nullptr;
     plan.need = p.splits > 1 ? (size_t)p.splits * (args ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float) : 0;
     // the fast staging path addresses a tile with 32-bit element offsets from the tile base
     const int64_t w_rows = (w_layout == MAM_W_MK) ? fwd::BM : fwd::KT;
-    p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30));
+    // (and the first k of every K range has to be 16-byte aligned)
+    p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30)) &&
+             (p.k_per_split % 4 == 0);
     // (16 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
     p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 25));
     // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
@@ -1112,10 +1162,11 @@ template <bool ARGS>
 static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                   const float *bias, float *c, int32_t *argmax, int32_t *argmin, float *w_sel, float *x_sel,
                   int64_t N, int64_t K, int64_t M, void *workspace, size_t workspace_size, void *stream,
-                  bool static_scratch = false)
+                  bool static_scratch = false, int64_t range_len = 0)
 {
     Plan plan;
-    int rc = make_plan(plan, ARGS, x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, x_sel, N, K, M);
+    int rc = make_plan(plan, ARGS, x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, w_sel, x_sel, N, K, M,
+                       range_len);
     if (rc != MAM_OK || N == 0 || M == 0) return rc;
     if (!x || !w || !c || (ARGS && (!argmax || !argmin)))
         return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
@@ -1153,7 +1204,15 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
         hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_KM, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
     rc = check_launch("mam_fwd_kernel");
     if (rc != MAM_OK) return rc;
-    if (p.splits > 1) {
+    if (p.splits > 1 && range_len > 0) {
+        // the caller's ranges are neurons of their own: resolve each and add them up
+        const unsigned mb = (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
+        if (w_layout == MAM_W_MK)
+            hipLaunchKernelGGL((mam_fwd_range_sum_kernel<MAM_W_MK, ARGS>), dim3(mb), dim3(256), 0, st, p);
+        else
+            hipLaunchKernelGGL((mam_fwd_range_sum_kernel<MAM_W_KM, ARGS>), dim3(mb), dim3(256), 0, st, p);
+        rc = check_launch("mam_fwd_range_sum_kernel");
+    } else if (p.splits > 1) {
         const unsigned mb = (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
         if (ARGS && p.coop)
             hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS, ARGS>), dim3(mb), dim3(256), 0, st, p);
@@ -1178,6 +1237,30 @@ static int launch_static(const float *x, int64_t ldx, const float *w, int64_t ld
 
 }  // namespace fwd
 }  // namespace mam
+
+extern "C" size_t mam_fc_forward_ranges_workspace(int64_t N, int64_t K, int64_t M, int64_t range_len, int with_indices)
+{
+    if (N <= 0 || K <= 0 || M <= 0 || range_len <= 0 || range_len >= K) return 0;
+    const size_t ranges = (size_t)((K + range_len - 1) / range_len);
+    return ranges * (with_indices ? 3 : 2) * (size_t)N * (size_t)M * sizeof(float);
+}
+
+extern "C" int mam_fc_forward_ranges(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                                     const float *bias, float *c, int32_t *argmax, int32_t *argmin, int64_t N,
+                                     int64_t K, int64_t M, int64_t range_len, void *workspace, size_t workspace_bytes,
+                                     void *stream)
+{
+    using namespace mam;
+    if (range_len <= 0) return fail(MAM_ERR_INVALID_ARGUMENT, "range_len must be positive");
+    if ((argmax == nullptr) != (argmin == nullptr))
+        return fail(MAM_ERR_INVALID_ARGUMENT, "argmax and argmin go together");
+    if (K > 0 && (K + range_len - 1) / range_len > 65535) return fail(MAM_ERR_UNSUPPORTED, "more than 65535 ranges");
+    if (argmax)
+        return fwd::launch<true>(x, ldx, w, ldw, w_layout, bias, c, argmax, argmin, nullptr, nullptr, N, K, M, workspace,
+                                 workspace_bytes, stream, false, range_len);
+    return fwd::launch<false>(x, ldx, w, ldw, w_layout, bias, c, nullptr, nullptr, nullptr, nullptr, N, K, M, workspace,
+                              workspace_bytes, stream, false, range_len);
+}
 
 extern "C" int mam_fc_forward_describe(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
                                        int64_t N, int64_t K, int64_t M, int with_indices, char *text, size_t text_bytes)

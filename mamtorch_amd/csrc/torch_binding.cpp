@@ -215,6 +215,55 @@ std::vector<at::Tensor> fullyconnected_wt_backward(const at::Tensor &a, const at
     return backward_impl(a, weight, MAM_W_MK, grad, argmax, argmin, sel);
 }
 
+// ---- the module's `splits`: consecutive K ranges, each a MAM neuron of its own, summed ----
+std::vector<at::Tensor> fullyconnected_ranges(const at::Tensor &a, const at::Tensor &weight,
+                                              const c10::optional<at::Tensor> &bias, int64_t range_len,
+                                              bool with_indices)
+{
+    const FwdShape s = check_forward(a, weight, MAM_W_MK, bias);
+    TORCH_CHECK(range_len > 0, "range_len must be positive");
+    const c10::DeviceGuard guard(a.device());
+    const int64_t ranges = std::max<int64_t>(1, (s.K + range_len - 1) / range_len);
+    auto c = at::empty({s.N, s.M}, a.options());
+    auto argmax = at::empty({with_indices ? ranges : 0, s.N, s.M}, a.options().dtype(at::kInt));
+    auto argmin = at::empty({with_indices ? ranges : 0, s.N, s.M}, a.options().dtype(at::kInt));
+    if (s.N == 0 || s.M == 0) return {c, argmax, argmin};
+    const size_t ws_bytes = mam_fc_forward_ranges_workspace(s.N, s.K, s.M, range_len, with_indices ? 1 : 0);
+    auto ws = workspace_for(ws_bytes, a);
+    check_rc(mam_fc_forward_ranges(a.data_ptr<float>(), row_stride(a, "a"), weight.data_ptr<float>(),
+                                   row_stride(weight, "weight"), MAM_W_MK, bias_ptr(bias), c.data_ptr<float>(),
+                                   with_indices ? argmax.data_ptr<int32_t>() : nullptr,
+                                   with_indices ? argmin.data_ptr<int32_t>() : nullptr, s.N, s.K, s.M, range_len,
+                                   ws.defined() ? ws.data_ptr() : nullptr, ws_bytes, current_stream(a)),
+             "mam_fc_forward_ranges");
+    return {c, argmax, argmin};
+}
+
+std::vector<at::Tensor> fullyconnected_ranges_backward(const at::Tensor &a, const at::Tensor &weight,
+                                                       const at::Tensor &grad, const at::Tensor &argmax,
+                                                       const at::Tensor &argmin, int64_t range_len)
+{
+    const FwdShape s = check_forward(a, weight, MAM_W_MK, c10::nullopt);
+    check_f32_2d(grad, "grad");
+    TORCH_CHECK(grad.size(0) == s.N && grad.size(1) == s.M, "grad must be (batch, out_features)");
+    TORCH_CHECK(range_len > 0, "range_len must be positive");
+    const int64_t ranges = std::max<int64_t>(1, (s.K + range_len - 1) / range_len);
+    for (const at::Tensor *t : {&argmax, &argmin})
+        TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kInt && t->is_contiguous() && t->dim() == 3 &&
+                        t->size(0) == ranges && t->size(1) == s.N && t->size(2) == s.M && t->device() == a.device(),
+                    "argmax / argmin must be contiguous int32 (ranges, batch, out_features) tensors on a's device");
+    const c10::DeviceGuard guard(a.device());
+    const at::Tensor g = grad.contiguous();
+    auto a_grad = at::empty({s.N, s.K}, a.options());
+    auto w_grad = at::empty(weight.sizes(), weight.options());
+    check_rc(mam_fc_backward_ranges(a.data_ptr<float>(), row_stride(a, "a"), weight.data_ptr<float>(),
+                                    row_stride(weight, "weight"), MAM_W_MK, g.data_ptr<float>(),
+                                    argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(), a_grad.data_ptr<float>(),
+                                    w_grad.data_ptr<float>(), s.N, s.K, s.M, range_len, current_stream(a)),
+             "mam_fc_backward_ranges");
+    return {a_grad, w_grad};
+}
+
 void selection_count(const at::Tensor &argmax, const at::Tensor &argmin, at::Tensor max_count,
                      at::Tensor min_count, int64_t mode)
 {
@@ -453,6 +502,8 @@ TORCH_LIBRARY(mamtorch_kernel_v4, m)
     m.def("fullyconnected_fast_wt(Tensor a, Tensor weight, Tensor? bias) -> Tensor");
     m.def("fullyconnected_wt_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin, Tensor? sel) -> Tensor[]");
     m.def("selection_count(Tensor argmax, Tensor argmin, Tensor(a!) max_count, Tensor(b!) min_count, int mode) -> ()");
+    m.def("fullyconnected_ranges(Tensor a, Tensor weight, Tensor? bias, int range_len, bool with_indices) -> Tensor[]");
+    m.def("fullyconnected_ranges_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin, int range_len) -> Tensor[]");
     m.def("blend(Tensor mam, Tensor mac, Tensor? bias, float alpha, float beta) -> Tensor");
     m.def("im2col(Tensor x, int k1, int k2, int s1, int s2) -> Tensor");
     m.def("col2im(Tensor cols, int B, int C, int H, int W, int k1, int k2, int s1, int s2) -> Tensor");
@@ -483,6 +534,8 @@ TORCH_LIBRARY_IMPL(mamtorch_kernel_v4, CUDA, m)
     m.impl("fullyconnected_fast_wt", &fullyconnected_fast_wt);
     m.impl("fullyconnected_wt_backward", &fullyconnected_wt_backward);
     m.impl("selection_count", &selection_count);
+    m.impl("fullyconnected_ranges", &fullyconnected_ranges);
+    m.impl("fullyconnected_ranges_backward", &fullyconnected_ranges_backward);
     m.impl("blend", &blend);
     m.impl("im2col", &im2col);
     m.impl("col2im", &col2im);

@@ -5,9 +5,62 @@ gather / scatter that feeds the MAM fully-connected kernel with convolution wind
 import torch
 from torch import Tensor
 
-__all__ = ["blend", "im2col", "col2im"]
+__all__ = ["blend", "im2col", "col2im", "fullyconnected_ranges"]
 
 K = torch.ops.mamtorch_kernel_v4
+
+
+def fullyconnected_ranges(a: Tensor, weight: Tensor, bias, range_len: int) -> Tensor:
+    """The module's `splits` as one operator: the inputs are cut into consecutive ranges of ``range_len``
+    (the last one shorter), every range is a MAM neuron of its own, and the result is the sum of the ranges'
+    max + min in ascending range order, then the bias.  a (N, in), weight (out, in) -> C (N, out).
+    Indices are only computed when a gradient will need them."""
+    with_indices = torch.is_grad_enabled() and (a.requires_grad or weight.requires_grad)
+    return K.fullyconnected_ranges.default(a, weight, bias, range_len, with_indices)[0]
+
+
+@torch.library.register_fake("mamtorch_kernel_v4::fullyconnected_ranges")
+def _(a, weight, bias, range_len, with_indices):
+    torch._check(a.dim() == 2 and weight.dim() == 2 and a.size(1) == weight.size(1))
+    torch._check(a.dtype == torch.float and weight.dtype == torch.float)
+    ranges = max(1, -(-a.size(1) // range_len)) if with_indices else 0
+    shape = (a.size(0), weight.size(0))
+    return [torch.empty(shape, dtype=torch.float, device=a.device),
+            torch.empty((ranges,) + shape, dtype=torch.int, device=a.device),
+            torch.empty((ranges,) + shape, dtype=torch.int, device=a.device)]
+
+
+@torch.library.register_fake("mamtorch_kernel_v4::fullyconnected_ranges_backward")
+def _(a, weight, grad, argmax, argmin, range_len):
+    torch._check(a.size(1) == weight.size(1) and grad.size(0) == a.size(0) and grad.size(1) == weight.size(0))
+    return [torch.empty(a.shape, dtype=torch.float, device=a.device),
+            torch.empty(weight.shape, dtype=torch.float, device=a.device)]
+
+
+def _ranges_setup(ctx, inputs, output):
+    a, weight, _, range_len, with_indices = inputs
+    _, argmax, argmin = output
+    need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+    ctx.range_len, ctx.with_indices = range_len, with_indices
+    ctx.save_for_backward(a if need else None, weight if need else None, argmax, argmin)
+
+
+def _ranges_backward(ctx, grad):
+    a, weight, argmax, argmin = ctx.saved_tensors
+    a_grad = w_grad = bias_grad = None
+    g = grad[0]
+    if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+        if not ctx.with_indices:
+            raise RuntimeError("fullyconnected_ranges was run without indices; its gradient needs them")
+        a_grad, w_grad = K.fullyconnected_ranges_backward.default(a, weight, g.contiguous(), argmax, argmin,
+                                                                  ctx.range_len)
+    if ctx.needs_input_grad[2]:
+        bias_grad = g.sum(dim=0)
+    return a_grad, w_grad, bias_grad, None, None
+
+
+torch.library.register_autograd("mamtorch_kernel_v4::fullyconnected_ranges", _ranges_backward,
+                                setup_context=_ranges_setup)
 
 
 def blend(mam: Tensor, mac: Tensor, bias, alpha: float, beta: float) -> Tensor:

@@ -170,19 +170,19 @@ class FullyConnected(Module):
 
         input_flat = input.reshape(-1, input.size()[-1])
         w = self._dropped_weight()
-        # the bias rides along in the kernel when nothing is added between MAM and bias (no MAC
-        # blend, no sum over splits), which keeps the reference's rounding order (max+min)+bias
-        fuse_bias = self.bias is not None and self.beta == 0 and self.splits == 1
-        fused = self.bias if fuse_bias else None
+        # without a MAC blend the bias rides along in the MAM kernel, after the sum of max and min (and
+        # after the sum over the splits): the reference's rounding order; with a blend the blend adds it
+        fuse_bias = self.bias is not None and self.beta == 0
+        fused = self.bias if fuse_bias and self.splits == 1 else None
+        fused_ranges = self.bias if fuse_bias else None
 
         if self.splits > 1:
-            sub, last = self.in_subfeatures, self.in_subfeatures_last
-            C_flat = self._mam_noargs(input_flat.narrow(-1, 0, sub), w.narrow(1, 0, sub), fused)
-            for i in range(1, self.splits - 1):
-                C_flat = C_flat + self._mam_noargs(input_flat.narrow(-1, i * sub, sub),
-                                                   w.narrow(1, i * sub, sub), None)
-            C_flat = C_flat + self._mam_noargs(input_flat.narrow(-1, self.in_features - last, last),
-                                               w.narrow(1, self.in_features - last, last), None)
+            # one operator for all slices: consecutive ranges of in_subfeatures inputs, summed in ascending
+            # order and then the bias -- the rounding order of the reference's `C_flat += ...` statements
+            if self.beta < 1:
+                C_flat = K.v4.fullyconnected_ranges(input_flat, w, fused_ranges, self.in_subfeatures)
+            else:
+                C_flat = torch.zeros((input_flat.shape[0], w.shape[0]), device=w.device, dtype=w.dtype)
         else:
             if self.store_args:
                 C_flat, argmax, argmin = K.v4.fullyconnected_wt(input_flat, w, fused)[:3]
@@ -195,8 +195,6 @@ class FullyConnected(Module):
             # alpha * MAM + beta * MAC + bias as one kernel, in the reference's rounding order
             mac_weight = self.weight.detach() if self.train_mam_only else self.weight
             C_flat = K.v4.blend(C_flat, F.linear(input_flat, mac_weight), self.bias, self.alpha, self.beta)
-        elif self.bias is not None and not fuse_bias:
-            C_flat = C_flat + self.bias.view(1, -1)
 
         C = C_flat.view(input.shape[:-1] + (self.weight.size(0),))
 
