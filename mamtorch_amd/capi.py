@@ -27,7 +27,7 @@ COUNT_FLAGS = 2
 EXPORTS = (
     "mam_version", "mam_error_string", "mam_last_error", "mam_init", "mam_set_option", "mam_device_info",
     "mam_fc_forward_static_limit", "mam_fc_forward_static", "mam_fc_forward_describe",
-    "mam_fc_forward_workspace", "mam_fc_forward",
+    "mam_fc_forward_workspace", "mam_fc_forward_workspace_for", "mam_fc_forward",
     "mam_fc_forward_values_workspace", "mam_fc_forward_values",
     "mam_fc_backward", "mam_selection_count",
     "mam_fc_forward_ranges_workspace", "mam_fc_forward_ranges", "mam_fc_backward_ranges",
@@ -56,6 +56,8 @@ def lib():
             fn = getattr(l, name)
             fn.restype = _size
             fn.argtypes = [_i64, _i64, _i64]
+        l.mam_fc_forward_workspace_for.restype = _size
+        l.mam_fc_forward_workspace_for.argtypes = [_i64, _i64, _i64, _int, _int]
         l.mam_fc_forward.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _i64,
                                      _i64, _i64, _ptr, _size, _ptr]
         l.mam_fc_forward_static_limit.restype = _size
@@ -132,7 +134,7 @@ def fc_forward(x, w, layout=W_KM, bias=None, workspace=None, w_sel=None, x_sel=N
     c = torch.empty((N, M), dtype=torch.float32, device=x.device)
     amax = torch.empty((N, M), dtype=torch.int32, device=x.device)
     amin = torch.empty((N, M), dtype=torch.int32, device=x.device)
-    need = l.mam_fc_forward_workspace(N, K, M)
+    need = l.mam_fc_forward_workspace_for(N, K, M, layout, 1)
     if workspace is None and need:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
@@ -160,7 +162,7 @@ def fc_forward_values(x, w, layout=W_KM, bias=None, workspace=None):
     l = lib()
     N, K, M = _dims(x, w, layout)
     c = torch.empty((N, M), dtype=torch.float32, device=x.device)
-    need = l.mam_fc_forward_values_workspace(N, K, M)
+    need = l.mam_fc_forward_workspace_for(N, K, M, layout, 0)
     if workspace is None and need:
         workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):

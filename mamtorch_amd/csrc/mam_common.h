@@ -35,6 +35,9 @@ int option(int which);
 // Compute units of the current device (read from the device at its set-up).
 int num_cus();
 
+// dst (cols, rows) contiguous = transpose of src (rows, cols), row stride ld.
+int transpose(const float *src, int64_t ld, float *dst, int64_t rows, int64_t cols, hipStream_t stream);
+
 // Two independent kernels of one call side by side: the first runs on a second stream of the library
 // (default priority, one per device) between a fork and a join event on the caller's stream.
 //   ForkedStream fork(st, units);      // decides; fork.side() is `st` itself when not forked

@@ -45,6 +45,62 @@ int fill_zero(void *ptr, int64_t count, hipStream_t stream)
     return check_launch("fill_zero_kernel");
 }
 
+// dst (cols, rows) contiguous = transpose of src (rows, cols) with row stride ld: 64 x 64 tiles through LDS,
+// 16-byte accesses on both sides when the shapes allow it.
+__global__ __launch_bounds__(256) void transpose_kernel(const float *__restrict__ src, int64_t ld,
+                                                        float *__restrict__ dst, int rows, int cols, int vec)
+{
+    __shared__ float tile[64][65];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = r0 + ty + 16 * i, c = c0 + tx * 4;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (r < rows) {
+            const float *row = src + (int64_t)r * ld;
+            if (vec && c + 3 < cols) {
+                v = *reinterpret_cast<const float4 *>(row + c);
+            } else {
+                if (c < cols) v.x = row[c];
+                if (c + 1 < cols) v.y = row[c + 1];
+                if (c + 2 < cols) v.z = row[c + 2];
+                if (c + 3 < cols) v.w = row[c + 3];
+            }
+        }
+        float *t = &tile[ty + 16 * i][tx * 4];
+        t[0] = v.x; t[1] = v.y; t[2] = v.z; t[3] = v.w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = c0 + ty + 16 * i, r = r0 + tx * 4;       // dst row c, dst columns r .. r + 3
+        if (c >= cols) continue;
+        float *out = dst + (int64_t)c * rows;
+        const float4 v = make_float4(tile[tx * 4][ty + 16 * i], tile[tx * 4 + 1][ty + 16 * i],
+                                     tile[tx * 4 + 2][ty + 16 * i], tile[tx * 4 + 3][ty + 16 * i]);
+        if (vec && r + 3 < rows && (rows & 3) == 0) {
+            *reinterpret_cast<float4 *>(out + r) = v;
+        } else {
+            if (r < rows) out[r] = v.x;
+            if (r + 1 < rows) out[r + 1] = v.y;
+            if (r + 2 < rows) out[r + 2] = v.z;
+            if (r + 3 < rows) out[r + 3] = v.w;
+        }
+    }
+}
+
+int transpose(const float *src, int64_t ld, float *dst, int64_t rows, int64_t cols, hipStream_t stream)
+{
+    if (rows <= 0 || cols <= 0) return MAM_OK;
+    const int64_t gx = ceil_div(cols, 64), gy = ceil_div(rows, 64);
+    if (gy > 65535 || gx > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "matrix too large for the transpose grid");
+    const int vec = (ld % 4 == 0) && ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0);
+    hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, stream, src, ld, dst,
+                       (int)rows, (int)cols, vec);
+    return check_launch("transpose_kernel");
+}
+
 namespace {
 struct DeviceState {
     std::mutex lock;             // set-up of this device, and its fork/join sequences

@@ -114,7 +114,7 @@ std::vector<at::Tensor> forward_impl(const at::Tensor &a, const at::Tensor &w, i
         if (with_sel) return {c, argmax, argmin, sel};
         return {c, argmax, argmin};
     }
-    const size_t ws_bytes = mam_fc_forward_workspace(s.N, s.K, s.M);
+    const size_t ws_bytes = mam_fc_forward_workspace_for(s.N, s.K, s.M, layout, 1);
     auto ws = workspace_for(ws_bytes, a);
     check_rc(mam_fc_forward(a.data_ptr<float>(), row_stride(a, "a"), w.data_ptr<float>(),
                             row_stride(w, "the weight operand"), layout, bias_ptr(bias),
@@ -133,7 +133,7 @@ at::Tensor forward_values_impl(const at::Tensor &a, const at::Tensor &w, int lay
     const c10::DeviceGuard guard(a.device());
     auto c = at::empty({s.N, s.M}, a.options());
     if (s.N == 0 || s.M == 0) return c;
-    const size_t ws_bytes = mam_fc_forward_values_workspace(s.N, s.K, s.M);
+    const size_t ws_bytes = mam_fc_forward_workspace_for(s.N, s.K, s.M, layout, 0);
     auto ws = workspace_for(ws_bytes, a);
     check_rc(mam_fc_forward_values(a.data_ptr<float>(), row_stride(a, "a"), w.data_ptr<float>(),
                                    row_stride(w, "the weight operand"), layout, bias_ptr(bias),

@@ -43,8 +43,10 @@ def _run_both_layouts(x, w_mk, bias=None, what=""):
     bd = None if bias is None else bias.to(dev)
     # the (M,K) layout twice: the library picks its wave-uniform-rows tiling where the shape allows it;
     # option MAM_FORWARD_TILING_WIDE keeps it on the first tiling
+    # the (K,M) operand twice as well: transposed once into the workspace and run on the (M,K) tilings where
+    # the shape allows it, and as it is on the general tiling
     for layout, w, tiling in ((capi.W_MK, w_mk.contiguous(), None), (capi.W_MK, w_mk.contiguous(), "wide"),
-                              (capi.W_KM, w_mk.T.contiguous(), None)):
+                              (capi.W_KM, w_mk.T.contiguous(), None), (capi.W_KM, w_mk.T.contiguous(), "wide")):
         wd = w.to(dev)
         with forward_tiling(tiling):
             c, amax, amin = capi.fc_forward(xd, wd, layout, bd)
