@@ -17,7 +17,11 @@
 // the entry is settled after the loop (first product equals the extreme: first entry, else second).
 // Measured, 4096 x 4096 weight at 10 % / 3 % / 1 % density, batch 256: 89 / 40 / 26 us against
 // 109 / 45 / 27 us with a compare and two selects per product; batch tiles of 64 rows per wave
-// instead of 256 were slower at all three (131 / 50 / 28 us).
+// instead of 256 were slower at all three (131 / 50 / 28 us); 4 or 16 entries in flight per buffer
+// instead of 8 changed nothing or spilled.  Timing-only builds at 10 %: the loads alone (arithmetic
+// removed) 95 us, the arithmetic alone (every load hitting one L1-resident row) 78 us, together
+// 90 us: the kernel sits on the vector memory path (1.7 GB of x values per call, half of them L1
+// hits, at about half of the path's 64 bytes per clock and CU) with the arithmetic hidden under it.
 // The lowest column missing from the row is found once per row; the
 // implicit-zero candidate x[n, missing] * 0 is compared last under the dense rule (greater wins,
 // equal -> lower index wins).  The 16 waves of a workgroup own 16 consecutive neurons and hand
@@ -73,7 +77,12 @@ __device__ __forceinline__ float lane_elem(const float4 &v, int t)
     return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w;
 }
 
-template <int TI>
+// LM (lane-held entry data): the row's column offsets and values are read 64 entries at a time by the
+// lanes of the wave (one coalesced load each, a block ahead of their use) and handed out with
+// v_readlane, instead of coming through the scalar cache group by group: the scalar loads sat on every
+// group's critical path, and their 64-bit address arithmetic took a third of the loop's instructions.
+// Needs the byte offset of every xT row to fit 32 bits.
+template <int TI, bool LM>
 __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
     const float *__restrict__ xT, int ldt, const int64_t *__restrict__ crow,
     const int64_t *__restrict__ col, const float *__restrict__ val, const float *__restrict__ bias,
@@ -128,18 +137,8 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
             amin[t] = 0.0f;
         }
 
-        // full groups of EG entries, software-pipelined: the loads of group g+1 are in flight while
-        // group g is consumed, so a row costs about one memory round trip per group
-        const int ng = nnz / EG;
         xvec xa[EG], xb[EG];
         float wa[EG], wb[EG];
-        auto issue = [&](int g, xvec (&xv)[EG], float (&wv)[EG]) {
-#pragma unroll
-            for (int u = 0; u < EG; ++u) {
-                xv[u] = *reinterpret_cast<const xvec *>(xl + ccol[beg + g * EG + u] * (int64_t)ldt);
-                wv[u] = cval[beg + g * EG + u];
-            }
-        };
         auto fold = [&](int pair, const xvec &x0, float w0, const xvec &x1, float w1) {
 #pragma unroll
             for (int t = 0; t < TI; ++t) {
@@ -158,6 +157,84 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
         auto consume = [&](int g, const xvec (&xv)[EG], const float (&wv)[EG]) {
 #pragma unroll
             for (int u = 0; u < EG; u += 2) fold(g * (EG / 2) + u / 2, xv[u], wv[u], xv[u + 1], wv[u + 1]);
+        };
+        // lowest column missing from the row: stored columns ascend, so it is the first position p
+        // with col[p] != p, or nnz when the row is a full prefix
+        int missing = nnz;
+        if (LM) {
+            static_assert(EG == 8, "the block loop below hands out 8 entries per group");
+            // entries past the end of the row repeat the last one: a repeated product never wins a strict
+            // compare, so every group is a whole group
+            const char *xbytes = reinterpret_cast<const char *>(xl);
+            const uint32_t row_bytes = (uint32_t)ldt * 4u;
+            uint32_t off_cur = 0, off_nxt = 0;     // lane e: byte offset of the xT row of entry 64 blk + e
+            float val_cur = 0.0f, val_nxt = 0.0f;
+            bool hole_found = false;
+            auto load_meta = [&](int blk, uint32_t &off, float &v) {
+                const int e = blk * 64 + lane;
+                const int ec = e < nnz ? e : nnz - 1;
+                const int64_t cc = col[beg + ec];
+                off = (uint32_t)cc * row_bytes;
+                v = val[beg + ec];
+                if (!hole_found) {
+                    const uint64_t mask = __ballot(e < nnz && cc != (int64_t)e);
+                    if (mask) { missing = blk * 64 + __builtin_ctzll(mask); hole_found = true; }
+                }
+            };
+            const int nblk = (nnz + 63) >> 6;
+            if (nblk > 0) load_meta(0, off_cur, val_cur);
+            // one group = 8 lanes' worth of (offset, value), read out of the block's registers
+#define MAM_CSR_ISSUE(G8, OFF, VAL, XV, WV)                                                                  \
+    _Pragma("unroll") for (int u = 0; u < EG; ++u) {                                                         \
+        const uint32_t so = __builtin_amdgcn_readlane(OFF, (G8) * EG + u);                                   \
+        WV[u] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, VAL), (G8) * EG + u)); \
+        XV[u] = *reinterpret_cast<const xvec *>(xbytes + so);                                                \
+    }
+            if (nblk > 0) { MAM_CSR_ISSUE(0, off_cur, val_cur, xa, wa) }
+            for (int blk = 0; blk < nblk; ++blk) {
+                const bool more = blk + 1 < nblk;
+                if (more) load_meta(blk + 1, off_nxt, val_nxt);
+                const int left = nnz - blk * 64;
+                const int ngb = left >= 64 ? 8 : (left + EG - 1) / EG;     // groups of this block
+                const int g0 = blk * 8;
+                // groups 0, 2, 4, 6 sit in buffer a, the odd ones in b; the loads of the next group are in
+                // flight while a group is consumed, across the block boundary too
+#define MAM_CSR_STEP(G8, XCUR, WCUR, XNXT, WNXT)                                                             \
+    if ((G8) < ngb) {                                                                                        \
+        if ((G8) + 1 < ngb) { MAM_CSR_ISSUE((G8) + 1, off_cur, val_cur, XNXT, WNXT) }                        \
+        __builtin_amdgcn_sched_barrier(0);                                                                   \
+        consume(g0 + (G8), XCUR, WCUR);                                                                      \
+        __builtin_amdgcn_sched_barrier(0);                                                                   \
+    }
+                MAM_CSR_STEP(0, xa, wa, xb, wb)
+                MAM_CSR_STEP(1, xb, wb, xa, wa)
+                MAM_CSR_STEP(2, xa, wa, xb, wb)
+                MAM_CSR_STEP(3, xb, wb, xa, wa)
+                MAM_CSR_STEP(4, xa, wa, xb, wb)
+                MAM_CSR_STEP(5, xb, wb, xa, wa)
+                MAM_CSR_STEP(6, xa, wa, xb, wb)
+                // the last group of a whole block: the first group of the next block goes out before it
+                if (7 < ngb) {
+                    if (more) { MAM_CSR_ISSUE(0, off_nxt, val_nxt, xa, wa) }
+                    __builtin_amdgcn_sched_barrier(0);
+                    consume(g0 + 7, xb, wb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                off_cur = off_nxt;
+                val_cur = val_nxt;
+            }
+#undef MAM_CSR_STEP
+#undef MAM_CSR_ISSUE
+        } else {
+        // full groups of EG entries, software-pipelined: the loads of group g+1 are in flight while
+        // group g is consumed, so a row costs about one memory round trip per group
+        const int ng = nnz / EG;
+        auto issue = [&](int g, xvec (&xv)[EG], float (&wv)[EG]) {
+#pragma unroll
+            for (int u = 0; u < EG; ++u) {
+                xv[u] = *reinterpret_cast<const xvec *>(xl + ccol[beg + g * EG + u] * (int64_t)ldt);
+                wv[u] = cval[beg + g * EG + u];
+            }
         };
         // two register buffers, the loop unrolled by two groups, so that no copy (which would
         // have to wait for the data) sits between issuing and consuming
@@ -181,15 +258,12 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
             const xvec x1 = *reinterpret_cast<const xvec *>(xl + ccol[beg + j] * (int64_t)ldt);
             fold(i / 2, x0, cval[beg + i], x1, cval[beg + j]);
         }
-
-        // lowest column missing from the row: stored columns ascend, so it is the first position p
-        // with col[p] != p, or nnz when the row is a full prefix
-        int missing = nnz;
         for (int base = 0; base < nnz; base += 64) {
             const int p = base + lane;
             const bool hole = p < nnz && col[beg + p] != (int64_t)p;
             const uint64_t mask = __ballot(hole);
             if (mask) { missing = base + __builtin_ctzll(mask); break; }
+        }
         }
         const bool has_zero = nnz < K;
         xvec zx;
@@ -459,10 +533,13 @@ static int g_bwd_lds_floats[kMaxDevices];
 
 static int setup_device(int dev)
 {
-    bool ok = hipFuncSetAttribute((const void *)csr_fwd_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  7 * ROWS * 64 * 4) == hipSuccess;
-    ok = hipFuncSetAttribute((const void *)csr_fwd_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                             7 * ROWS * 256 * 4) == hipSuccess && ok;
+    bool ok = true;
+    const void *small[] = {(const void *)csr_fwd_kernel<1, false>, (const void *)csr_fwd_kernel<1, true>};
+    const void *large[] = {(const void *)csr_fwd_kernel<4, false>, (const void *)csr_fwd_kernel<4, true>};
+    for (const void *k : small)
+        ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 7 * ROWS * 64 * 4) == hipSuccess && ok;
+    for (const void *k : large)
+        ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 7 * ROWS * 256 * 4) == hipSuccess && ok;
     if (!ok) {
         (void)hipGetLastError();
         return fail(MAM_ERR_LAUNCH, "could not raise the LDS limit of the CSR forward kernels");
@@ -540,18 +617,21 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
     const int vec_out = (M % 4 == 0) && ((uintptr_t)c % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
                         ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)w_sel % 16 == 0) &&
                         ((uintptr_t)pos_sel % 16 == 0);
-    if (N <= 64) {
-        hipLaunchKernelGGL((csr::csr_fwd_kernel<1>), dim3((unsigned)ceil_div(M, csr::ROWS), 1u), dim3(csr::NT_F),
-                           (size_t)7 * csr::ROWS * 64 * sizeof(float),
-                           st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel, pos_sel, (int)N,
-                           (int)K, (int)M, vec_out);
-    } else {
-        const int64_t gy = ceil_div(N, 256);
-        if (gy > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the CSR forward grid");
-        hipLaunchKernelGGL((csr::csr_fwd_kernel<4>), dim3((unsigned)ceil_div(M, csr::ROWS), (unsigned)gy),
-                           dim3(csr::NT_F), (size_t)7 * csr::ROWS * 256 * sizeof(float), st, xT, (int)ldt, crow, col, val, bias, c, argmax, argmin, w_sel,
-                           pos_sel, (int)N, (int)K, (int)M, vec_out);
-    }
+    // the lane-held entry data needs every xT row's byte offset in 32 bits
+    const bool lm = (int64_t)K * ldt * 4 < ((int64_t)1 << 32);
+    const dim3 grid1((unsigned)ceil_div(M, csr::ROWS), 1u);
+    const int64_t gy = ceil_div(N, 256);
+    if (gy > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the CSR forward grid");
+    const dim3 grid4((unsigned)ceil_div(M, csr::ROWS), (unsigned)gy);
+    const size_t lds1 = (size_t)7 * csr::ROWS * 64 * sizeof(float), lds4 = (size_t)7 * csr::ROWS * 256 * sizeof(float);
+#define MAM_CSR_LAUNCH(TI, LM, GRID, LDS)                                                                           \
+    hipLaunchKernelGGL((csr::csr_fwd_kernel<TI, LM>), GRID, dim3(csr::NT_F), LDS, st, xT, (int)ldt, crow, col, val, \
+                       bias, c, argmax, argmin, w_sel, pos_sel, (int)N, (int)K, (int)M, vec_out)
+    if (N <= 64 && lm) MAM_CSR_LAUNCH(1, true, grid1, lds1);
+    else if (N <= 64) MAM_CSR_LAUNCH(1, false, grid1, lds1);
+    else if (lm) MAM_CSR_LAUNCH(4, true, grid4, lds4);
+    else MAM_CSR_LAUNCH(4, false, grid4, lds4);
+#undef MAM_CSR_LAUNCH
     return check_launch("csr_fwd_kernel");
 }
 
