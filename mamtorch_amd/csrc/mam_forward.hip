@@ -771,7 +771,8 @@ __global__ __launch_bounds__(256) void mam_fwd_range_sum_kernel(const Params p)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Second tiling for the (M,K) layout with whole 64-k tiles: batch rows are wave-uniform.
+// Second tiling for the (M,K) layout with K a multiple of 16 (64-k tiles, the last one may hold one to
+// three 16-k groups): batch rows are wave-uniform.
 //
 // A wave owns 4 batch rows x 128 neurons (lane + 64 j): its x operands are the same for all
 // lanes, so they come through the scalar cache into SGPRs (a VALU multiply takes one SGPR
@@ -816,7 +817,9 @@ constexpr int BM_MAX = Cfg<2>::BM;
 
 typedef const __attribute__((address_space(4))) float const_f32;
 
-template <int TJ, bool ARGS, bool SPLIT>
+// TAIL: K (or the last K range) is a multiple of G = 16 but not of 64; the last tile is partial.  A separate
+// instantiation, so that the whole-tile kernel stays exactly what it was.
+template <int TJ, bool ARGS, bool SPLIT, bool TAIL>
 __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 {
     using C = sx::Cfg<TJ>;
@@ -842,7 +845,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     const int row0 = tn * sx::BN + sx::TI * wave, col0 = tm * C::BM;
     const int kb = split * p.k_per_split;
     const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
-    const int ntiles = (ke - kb) / sx::KT;    // the host sends only whole tiles here
+    const int ntiles = (ke - kb) / sx::KT;    // whole tiles; a rest of whole 16-k groups follows as a partial tile
 
     float vmax[sx::TI][TJ], vmin[sx::TI][TJ];
     int gmax[sx::TI][TJ], gmin[sx::TI][TJ];
@@ -887,9 +890,16 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
                                              (__attribute__((address_space(3))) void *)(tile + inst * 256), 16, 0, 0);
         }
     };
+    // The last tile of a K range that is not a multiple of 64 (but of G = 16): only its whole groups are
+    // loaded (lanes whose 16-byte chunk lies past the range are switched off, so nothing past the end of a
+    // weight row is read) and only they are computed.
+    const int tail_groups = TAIL ? ((ke - kb) % sx::KT) / G : 0;
+    const int nt_all = ntiles + (tail_groups ? 1 : 0);
     auto compute = [&](const float *tile, int t) {
+        const int ng = (TAIL && t == ntiles) ? tail_groups : sx::KT / G;
 #pragma unroll
         for (int gg = 0; gg < sx::KT / G; ++gg) {
+            if (TAIL && gg >= ng) break;
             const int grel = t * (sx::KT / G) + gg;
             float xv[sx::TI][G];
 #pragma unroll
@@ -925,19 +935,36 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
             }
         }
     };
+    auto dma_any = [&](const char *wk, float *tile, int t) {
+        if (!TAIL || t < ntiles) {
+            dma(wk, tile);
+        } else {
+#pragma unroll
+            for (int u = 0; u < C::DMA_PER_WAVE; ++u) {
+                const int inst = wave + (sx::NT / 64) * u;
+                const int r = inst * (64 / sx::CHUNKS) + lane / sx::CHUNKS;
+                const int chunk = (lane % sx::CHUNKS) ^ ((r / sx::RPB) & (sx::CHUNKS - 1));
+                if (chunk * 4 < tail_groups * G) {
+                    const char *src = wk + (uint64_t)doff[u * sx::NT];
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                                     (__attribute__((address_space(3))) void *)(tile + inst * 256), 16, 0, 0);
+                }
+            }
+        }
+    };
 
     const char *wk = reinterpret_cast<const char *>(p.w + (int64_t)col0 * p.ldw + kb);
-    if (ntiles > 0) {
-        dma(wk, tile_a);
+    if (nt_all > 0) {
+        dma_any(wk, tile_a, 0);
         __syncthreads();
-        for (int t = 0; t < ntiles; t += 2) {
+        for (int t = 0; t < nt_all; t += 2) {
             wk += sx::KT * sizeof(float);
-            if (t + 1 < ntiles) dma(wk, tile_b);
+            if (t + 1 < nt_all) dma_any(wk, tile_b, t + 1);
             compute(tile_a, t);
             __syncthreads();
-            if (t + 1 >= ntiles) break;
+            if (t + 1 >= nt_all) break;
             wk += sx::KT * sizeof(float);
-            if (t + 2 < ntiles) dma(wk, tile_a);
+            if (t + 2 < nt_all) dma_any(wk, tile_a, t + 2);
             compute(tile_b, t + 1);
             __syncthreads();
         }
@@ -1123,12 +1150,12 @@ static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const f
     p.N = (int)N; p.K = (int)K; p.M = (int)M;
     p.vec_x = (ldx % 4 == 0) && ((uintptr_t)x % 16 == 0);
     p.vec_w = (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0);
-    // The wave-uniform-rows tiling takes (M,K) weights with aligned rows and whole 64-k tiles; option
+    // The wave-uniform-rows tiling takes (M,K) weights with aligned rows and K a multiple of 16; option
     // MAM_OPT_FORWARD_TILING = MAM_FORWARD_TILING_WIDE keeps every shape on the first tiling (for
     // comparisons and tests).
     // (range_len > 0: the caller fixes the K ranges -- the module's `splits` -- instead of the launch
     // heuristics; the wave-uniform-rows tiling then also needs whole 64-k tiles per range)
-    const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % sx::KT == 0) &&
+    const bool use_sx = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) &&
                         (range_len % sx::KT == 0) && (ldw * sx::BM_MAX < (1ll << 30)) &&
                         option(MAM_OPT_FORWARD_TILING) != MAM_FORWARD_TILING_WIDE;
     plan.use_sx = use_sx;
@@ -1231,10 +1258,15 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
         if (rc != MAM_OK) return rc;
         p.w = wt;
     }
-    if (use_sx && p.splits > 1)
-        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+    const bool tail = K % sx::KT != 0;
+    if (use_sx && p.splits > 1 && tail)
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+    else if (use_sx && p.splits > 1)
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+    else if (use_sx && tail)
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, false, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (use_sx)
-        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, false, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (w_layout == MAM_W_MK)
         hipLaunchKernelGGL((mam_fwd_kernel<MAM_W_MK, ARGS>), dim3((unsigned)nblk), dim3(NT), 0, st, p);
     else
@@ -1280,7 +1312,7 @@ extern "C" size_t mam_fc_forward_workspace_for(int64_t N, int64_t K, int64_t M, 
     if (N <= 0 || K <= 0 || M <= 0) return 0;
     size_t bytes = mam::fwd::workspace_bytes(N, K, M, with_indices != 0);
     // room for the transposed copy of a (K, M) operand (see launch); without it the call still works
-    if (w_layout == MAM_W_KM && K % mam::fwd::sx::KT == 0 && mam::fwd::transposed_operand_pays(N, K, M))
+    if (w_layout == MAM_W_KM && K % mam::fwd::G == 0 && mam::fwd::transposed_operand_pays(N, K, M))
         bytes += ((size_t)M * (size_t)K * sizeof(float) + 255) / 256 * 256;
     return bytes;
 }

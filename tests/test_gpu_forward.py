@@ -169,6 +169,28 @@ def test_ragged_batch_and_neurons_on_whole_k_tiles(shape):
     _run_both_layouts(x, w, bias, "whole k tiles %s" % (shape,))
 
 
+@pytest.mark.parametrize("shape", [(1, 16, 1), (33, 48, 130), (70, 208, 300), (64, 784, 256), (31, 1072, 127),
+                                   (257, 4112, 129), (40, 8240, 260), (256, 4144, 512)])
+def test_partial_last_k_tile(shape):
+    """K a multiple of 16 but not of 64: the wave-uniform-rows tiling ends on a partial tile of one, two or
+    three 16-k groups, alone (K < 64), after whole tiles, and at the end of the last range of a split K.  The
+    second case plants the extremes inside that partial tile and ties them with earlier columns."""
+    N, K, M = shape
+    x, w, _ = random_case(N, K, M, seed=N + K, w_scale=1.0 / K ** 0.5)
+    bias = torch.randn(M, generator=torch.Generator().manual_seed(K))
+    _run_both_layouts(x, w, bias, "partial tile %s" % (shape,))
+    x2, w2 = x.clone(), w.clone()
+    tail0 = K - K % 64
+    x2[:, K - 1] = 50.0
+    w2[:, K - 1] = torch.where(torch.arange(M) % 2 == 0, 1.0, -1.0)
+    x2[:, tail0] = 50.0
+    w2[:, tail0] = w2[:, K - 1]
+    if tail0 >= 64:
+        x2[N // 2:, 3] = 50.0
+        w2[:, 3] = w2[:, K - 1]
+    _run_both_layouts(x2, w2, None, "partial tile, planted %s" % (shape,))
+
+
 def test_aligned_views_with_longer_rows_on_whole_k_tiles():
     """Aligned 128-k windows of wider x and weight matrices (module splits > 1): row strides exceed K."""
     from mamtorch_amd import capi

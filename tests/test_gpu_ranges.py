@@ -30,7 +30,8 @@ def _oracle_ranges(x, w_mk, bias, range_len):
 
 @pytest.mark.parametrize("N,K,M,range_len", [(256, 4096, 512, 1024), (96, 2048, 200, 512), (70, 123, 45, 41),
                                              (33, 100, 20, 34), (64, 784, 256, 262), (40, 300, 70, 300),
-                                             (17, 64, 33, 16), (300, 1536, 640, 768)])
+                                             (17, 64, 33, 16), (300, 1536, 640, 768), (64, 784, 256, 256),
+                                             (50, 1072, 130, 512)])
 def test_forward_and_backward_over_ranges(N, K, M, range_len):
     from mamtorch_amd import capi
 
