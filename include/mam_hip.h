@@ -261,6 +261,16 @@ int mam_blend(const float *mam_out, const float *mac_out, const float *bias, flo
               int64_t N, int64_t M, void *stream);
 
 /*
+ * out (M, K) contiguous = w (M, K, row stride ldw) * (keep ? 1 : 0), keep (M, K) contiguous bytes: the
+ * training-time weight dropout of the module (mamtorch/nn/v4/fullyconnected.py:143-148, there a float
+ * Bernoulli mask of the weight's size times the transposed weight) in one pass from a byte mask.  The
+ * product is formed as the reference forms it, so a dropped weight is a zero with the weight's sign.  The
+ * same call masks the weight gradient on the way back.
+ */
+int mam_apply_keep(const float *w, int64_t ldw, const unsigned char *keep, float *out, int64_t M, int64_t K,
+                   void *stream);
+
+/*
  * MAM convolution as the MAM fully-connected kernel over gathered windows.  x is (B, C, H, W) contiguous
  * (a 1-D convolution has H = k1 = s1 = 1), windows are k1 x k2 with strides s1, s2 and no padding (the
  * caller pads, as the reference's modules do), output positions L1 = (H - k1) / s1 + 1, L2 likewise.

@@ -33,7 +33,7 @@ EXPORTS = (
     "mam_fc_forward_ranges_workspace", "mam_fc_forward_ranges", "mam_fc_backward_ranges",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward", "mam_csr_validate",
     "mam_csr_spmm", "mam_coo_spmm",
-    "mam_blend", "mam_im2col", "mam_col2im",
+    "mam_blend", "mam_apply_keep", "mam_im2col", "mam_col2im",
     "mam_prune_row_offsets", "mam_prune_fill_csr", "mam_prune_apply",
 )
 
@@ -83,6 +83,7 @@ def lib():
         l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                           _ptr, _i64, _i64, _i64, _i64, _ptr]
         l.mam_blend.argtypes = [_ptr, _ptr, _ptr, ctypes.c_float, ctypes.c_float, _ptr, _i64, _i64, _ptr]
+        l.mam_apply_keep.argtypes = [_ptr, _i64, _ptr, _ptr, _i64, _i64, _ptr]
         l.mam_im2col.argtypes = [_ptr, _ptr] + [_i64] * 8 + [_ptr]
         l.mam_col2im.argtypes = [_ptr, _ptr] + [_i64] * 8 + [_ptr]
         l.mam_csr_validate.argtypes = [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr]

@@ -5,6 +5,8 @@
 //  * mam_blend: out = (alpha * mam + beta * mac) + bias, the module's MAC blend
 //    (mamtorch/nn/v4/fullyconnected.py:190-198) in one pass and in the reference's rounding order
 //    (two products, their sum, then the bias; no fused multiply-add).
+//  * mam_apply_keep: the training-time weight dropout (mamtorch/nn/v4/fullyconnected.py:143-148) from a
+//    byte mask, one pass over the weight.
 //  * mam_im2col / mam_col2im: the reference's retired MAM convolutions
 //    (mamtorch/kernel/backup/mamconv1d_forward.txt:26-166, mamconv2d_forward.txt) run the MAM reduction
 //    over the window positions and channels of each output position, with the index
@@ -42,6 +44,40 @@ __global__ __launch_bounds__(256) void blend_kernel(const float *__restrict__ ma
             float r = alpha * mam[i] + beta * mac[i];
             if (bias) r = r + bias[i % M];
             out[i] = r;
+        }
+    }
+}
+
+// out[m][k] = w[m][k] * (keep[m][k] ? 1 : 0): the training-time weight dropout of the module
+// (mamtorch/nn/v4/fullyconnected.py:143-148: `weight * bernoulli mask`) with the mask as one byte per
+// weight.  The product keeps the reference's bits: a dropped weight becomes a zero with the weight's sign,
+// and a non-finite one becomes NaN.
+__global__ __launch_bounds__(256) void keep_kernel(const float *__restrict__ w, int64_t ldw,
+                                                   const unsigned char *__restrict__ keep,
+                                                   float *__restrict__ out, int64_t M, int K, int vec)
+{
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    if (vec) {
+        const int qpr = K >> 2;                   // quads per row
+        const int64_t quads = M * (int64_t)qpr;
+        for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += stride) {
+            const int64_t m = q / qpr;
+            const int k = (int)(q - m * qpr) << 2;
+            const float4 a = *reinterpret_cast<const float4 *>(w + m * ldw + k);
+            const uint32_t kb = *reinterpret_cast<const uint32_t *>(keep + m * K + k);
+            float4 r;
+            r.x = a.x * ((kb & 0xffu) ? 1.0f : 0.0f);
+            r.y = a.y * ((kb & 0xff00u) ? 1.0f : 0.0f);
+            r.z = a.z * ((kb & 0xff0000u) ? 1.0f : 0.0f);
+            r.w = a.w * ((kb & 0xff000000u) ? 1.0f : 0.0f);
+            *reinterpret_cast<float4 *>(out + m * K + k) = r;
+        }
+    } else {
+        const int64_t total = M * (int64_t)K;
+        for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+            const int64_t m = i / K;
+            const int k = (int)(i - m * K);
+            out[i] = w[m * ldw + k] * (keep[i] ? 1.0f : 0.0f);
         }
     }
 }
@@ -170,6 +206,25 @@ extern "C" int mam_blend(const float *mam_out, const float *mac_out, const float
     hipLaunchKernelGGL(module::blend_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                        mam_out, mac_out, bias, alpha, beta, out, total, (int)M, vec);
     return check_launch("blend_kernel");
+}
+
+extern "C" int mam_apply_keep(const float *w, int64_t ldw, const unsigned char *keep, float *out, int64_t M,
+                              int64_t K, void *stream)
+{
+    using namespace mam;
+    if (M < 0 || K < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
+    if (M == 0 || K == 0) return MAM_OK;
+    if (!w || !keep || !out) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    if (ldw < K) return fail(MAM_ERR_INVALID_ARGUMENT, "leading dimension smaller than the row length");
+    if (K > INT32_MAX / 2 || M > INT32_MAX / 2) return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
+    const int vec = (K % 4 == 0) && (ldw % 4 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0) &&
+                    ((uintptr_t)keep % 4 == 0);
+    const int64_t total = M * K;
+    int64_t blocks = ceil_div(vec ? total / 4 : total, 256);
+    if (blocks > 16 * num_cus()) blocks = 16 * num_cus();
+    hipLaunchKernelGGL(module::keep_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream), w,
+                       ldw, keep, out, M, (int)K, vec);
+    return check_launch("keep_kernel");
 }
 
 extern "C" int mam_im2col(const float *x, float *cols, int64_t B, int64_t C, int64_t H, int64_t W, int64_t k1,

@@ -307,6 +307,24 @@ at::Tensor blend(const at::Tensor &mam, const at::Tensor &mac, const c10::option
     return out;
 }
 
+// weight (out, in) times a {0, 1} mask kept as bool / uint8: the module's weight dropout and its gradient
+at::Tensor apply_keep(const at::Tensor &w, const at::Tensor &keep)
+{
+    check_f32_2d(w, "weight");
+    TORCH_CHECK(keep.is_cuda() && (keep.scalar_type() == at::kBool || keep.scalar_type() == at::kByte) &&
+                    keep.sizes() == w.sizes() && keep.is_contiguous(),
+                "keep must be a contiguous bool or uint8 GPU tensor of the weight's shape");
+    check_same_device(w, keep, "keep");
+    const c10::DeviceGuard guard(w.device());
+    const at::Tensor wc = (w.stride(1) == 1 && w.stride(0) >= w.size(1)) || w.numel() == 0 ? w : w.contiguous();
+    auto out = at::empty({w.size(0), w.size(1)}, w.options());
+    if (out.numel() > 0)
+        check_rc(mam_apply_keep(wc.data_ptr<float>(), wc.stride(0), static_cast<const unsigned char *>(keep.data_ptr()),
+                                out.data_ptr<float>(), w.size(0), w.size(1), current_stream(w)),
+                 "mam_apply_keep");
+    return out;
+}
+
 at::Tensor im2col(const at::Tensor &x, int64_t k1, int64_t k2, int64_t s1, int64_t s2)
 {
     TORCH_CHECK(x.is_cuda() && x.scalar_type() == at::kFloat && x.dim() == 4, "x must be a float32 GPU tensor (B, C, H, W)");
@@ -505,6 +523,7 @@ TORCH_LIBRARY(mamtorch_kernel_v4, m)
     m.def("fullyconnected_ranges(Tensor a, Tensor weight, Tensor? bias, int range_len, bool with_indices) -> Tensor[]");
     m.def("fullyconnected_ranges_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin, int range_len) -> Tensor[]");
     m.def("blend(Tensor mam, Tensor mac, Tensor? bias, float alpha, float beta) -> Tensor");
+    m.def("apply_keep(Tensor weight, Tensor keep) -> Tensor");
     m.def("im2col(Tensor x, int k1, int k2, int s1, int s2) -> Tensor");
     m.def("col2im(Tensor cols, int B, int C, int H, int W, int k1, int k2, int s1, int s2) -> Tensor");
 }
@@ -537,6 +556,7 @@ TORCH_LIBRARY_IMPL(mamtorch_kernel_v4, CUDA, m)
     m.impl("fullyconnected_ranges", &fullyconnected_ranges);
     m.impl("fullyconnected_ranges_backward", &fullyconnected_ranges_backward);
     m.impl("blend", &blend);
+    m.impl("apply_keep", &apply_keep);
     m.impl("im2col", &im2col);
     m.impl("col2im", &col2im);
 }

@@ -5,7 +5,7 @@ gather / scatter that feeds the MAM fully-connected kernel with convolution wind
 import torch
 from torch import Tensor
 
-__all__ = ["blend", "im2col", "col2im", "fullyconnected_ranges"]
+__all__ = ["blend", "apply_keep", "im2col", "col2im", "fullyconnected_ranges"]
 
 K = torch.ops.mamtorch_kernel_v4
 
@@ -68,6 +68,13 @@ def blend(mam: Tensor, mac: Tensor, bias, alpha: float, beta: float) -> Tensor:
     return K.blend.default(mam, mac, bias, float(alpha), float(beta))
 
 
+def apply_keep(weight: Tensor, keep: Tensor) -> Tensor:
+    """weight (out, in) * keep, keep a bool / uint8 mask of the same shape: the weight dropout of
+    ``FullyConnected`` (mamtorch/nn/v4/fullyconnected.py:143-148) in one pass; its gradient is the same
+    masking of the incoming gradient."""
+    return K.apply_keep.default(weight, keep)
+
+
 def im2col(x: Tensor, k1: int, k2: int, s1: int, s2: int) -> Tensor:
     """x (B, C, H, W) -> (B * L1 * L2, k2 * k1 * C) windows, column (j2 * k1 + j1) * C + c."""
     return K.im2col.default(x, k1, k2, s1, s2)
@@ -99,6 +106,24 @@ def _blend_backward(ctx, grad):
 
 
 torch.library.register_autograd("mamtorch_kernel_v4::blend", _blend_backward, setup_context=_blend_setup)
+
+
+@torch.library.register_fake("mamtorch_kernel_v4::apply_keep")
+def _(weight, keep):
+    torch._check(weight.dim() == 2 and weight.dtype == torch.float and keep.shape == weight.shape)
+    return torch.empty(weight.shape, dtype=torch.float, device=weight.device)
+
+
+def _keep_setup(ctx, inputs, output):
+    ctx.save_for_backward(inputs[1])
+
+
+def _keep_backward(ctx, grad):
+    (keep,) = ctx.saved_tensors
+    return K.apply_keep.default(grad, keep), None
+
+
+torch.library.register_autograd("mamtorch_kernel_v4::apply_keep", _keep_backward, setup_context=_keep_setup)
 
 
 def _out_positions(H, W, k1, k2, s1, s2):

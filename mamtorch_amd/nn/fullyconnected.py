@@ -151,10 +151,11 @@ class FullyConnected(Module):
         if self.training and self.wdrop_rate != 0:
             if not (0 < self.wdrop_rate < 1):
                 raise Exception("wdrop_rate must be between 0 and 1.")
-            # the mask is drawn in (in, out) order, as the reference draws it on weight.T
-            keep = torch.bernoulli(torch.full((self.in_features, self.out_features), 1 - self.wdrop_rate,
-                                              dtype=w.dtype, device=w.device))
-            w = w * keep.T
+            # the reference draws a float mask of the weight's size and multiplies (a second copy of W and
+            # three more passes over it); here the mask is one byte per weight, drawn by torch's generator,
+            # and one kernel forms weight * mask; autograd masks the weight gradient with the same call
+            keep = torch.empty(w.shape, dtype=torch.bool, device=w.device).bernoulli_(1 - self.wdrop_rate)
+            w = K.v4.apply_keep(w, keep)
         return w
 
     def _mam_noargs(self, x: Tensor, w: Tensor, bias) -> Tensor:

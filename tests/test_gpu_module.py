@@ -67,6 +67,8 @@ def test_opcheck():
     _, amax, amin = torch.ops.mamtorch_kernel_v4.fullyconnected(a.detach(), b.detach())
     torch.library.opcheck(torch.ops.mamtorch_kernel_v4.fullyconnected_backward,
                           (a.detach(), b.detach(), grad.to(DEV), amax, amin), test_utils=("test_schema", "test_faketensor"))
+    keep = torch.rand(11, 37, device=DEV) < 0.5
+    torch.library.opcheck(torch.ops.mamtorch_kernel_v4.apply_keep, (wt, keep), test_utils=tests)
 
 
 def test_operator_errors_are_runtime_errors():
@@ -190,6 +192,60 @@ def test_module_weight_dropout_and_output_dropout_run():
     layer.wdrop_rate = 1.5
     with pytest.raises(Exception, match="wdrop_rate must be between 0 and 1"):
         layer(x.to(DEV))
+
+
+@pytest.mark.parametrize("shape", [(6, 20), (45, 123), (256, 784), (130, 4096)])
+def test_apply_keep_is_the_reference_expression_on_a_fixed_mask(shape):
+    """weight * mask with the mask as bytes: bit-equal to the reference's float expression
+    (mamtorch/nn/v4/fullyconnected.py:143-148), signed zeros and non-finite weights included; strided weight
+    views; the gradient is the same masking."""
+    M, Kin = shape
+    g = torch.Generator().manual_seed(M + Kin)
+    w = torch.randn(M, Kin, generator=g)
+    w[0, 0], w[M - 1, Kin - 1], w[M // 2, 1] = float("inf"), -0.0, float("nan")
+    keep = torch.rand(M, Kin, generator=g) < 0.6
+    keep[0, 0] = True
+    w[1, 2], keep[1, 2] = float("-inf"), False      # inf * 0: NaN here as in the reference (its sign is the platform's)
+    want = w * keep.to(torch.float32)
+    wd = w.to(DEV).requires_grad_(True)
+    got = mt.kernel.v4.apply_keep(wd, keep.to(DEV))
+    assert torch.isnan(got[1, 2]) and torch.isnan(want[1, 2])
+    want[1, 2] = got[1, 2].item()
+    want = torch.where(torch.isnan(want), got.detach().cpu(), want)
+    assert torch.isnan(got[M // 2, 1])
+    assert_bits_equal(got.detach().cpu().numpy(), want.numpy(), "apply_keep %s" % (shape,))
+    grad = torch.randn(M, Kin, generator=g)
+    got.backward(grad.to(DEV))
+    assert_bits_equal(wd.grad.cpu().numpy(), (grad * keep.to(torch.float32)).numpy(), "apply_keep gradient")
+    # a view with a longer row stride and an unaligned base
+    wide = torch.randn(M, Kin + 7, generator=g).to(DEV)
+    got = mt.kernel.v4.apply_keep(wide[:, 3:3 + Kin], keep.to(DEV))
+    assert_bits_equal(got.cpu().numpy(), (wide[:, 3:3 + Kin].cpu() * keep.to(torch.float32)).numpy(), "strided view")
+    got8 = mt.kernel.v4.apply_keep(wd.detach(), keep.to(DEV).to(torch.uint8))
+    assert_bits_equal(got8.cpu().numpy(), want.numpy(), "uint8 mask")
+
+
+def test_module_weight_dropout_against_the_oracle():
+    """Training-time weight dropout: the layer's output is the MAM of x and weight * mask for the mask the
+    layer drew (same generator state, same call), bit for bit; dropped weights get no gradient."""
+    x, w, grad = random_case(33, 128, 40, seed=17)
+    layer = _layer_from(w, None, wdrop_rate=0.3).train()
+    torch.manual_seed(5)
+    y = layer(x.to(DEV))
+    torch.manual_seed(5)
+    keep = torch.empty(w.shape, dtype=torch.bool, device=DEV).bernoulli_(1 - 0.3)
+    assert 0.5 < keep.float().mean().item() < 0.9
+    wm = (w * keep.cpu().to(torch.float32))
+    want = oracle.forward(x.numpy(), wm.numpy(), oracle.W_MK)
+    assert_bits_equal(y.detach().cpu().numpy(), want[0], "weight dropout y")
+    y.backward(grad.to(DEV))
+    _, wo = oracle.backward(x.numpy(), wm.numpy(), grad.numpy(), want[1], want[2], oracle.W_MK)
+    wo = wo * keep.cpu().numpy()
+    np.testing.assert_allclose(layer.weight.grad.cpu().numpy(), wo, rtol=1e-5, atol=1e-6)
+    assert (layer.weight.grad[~keep] == 0).all()
+    layer.eval()
+    y = layer(x.to(DEV))
+    assert_bits_equal(y.detach().cpu().numpy(), oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)[0], "eval: no dropout")
 
 
 def test_sparse_operator_and_autograd_function():
