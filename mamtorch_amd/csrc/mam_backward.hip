@@ -49,80 +49,216 @@ __device__ __forceinline__ void lds_add_sparse(float *addr, float v)
     if (!done) lds_add(addr, v);
 }
 
+// ---- exact accumulation of x_grad in 64-bit fixed point ------------------------------------------------
+// An fp32 term is m * 2^(e - 150) with a 24-bit integer m.  Relative to a window [e_lo, e_lo + span) of
+// biased exponents it is the integer m << (e - e_lo), and integer adds are exact and commute: the cell ends
+// up with the exact sum of its terms whatever order the lanes arrive in, rounded to fp32 once when the slab
+// is stored -- and the integer LDS atomic costs ~8 cycles per 64-lane instruction where ds_add_f32 costs
+// ~190.  span leaves room for every term a cell can receive (2 * M * planes), so the sum cannot overflow.
+// The window is placed by the largest term of the workgroup's first trip (plus 4 binades where that is
+// not the whole row).  The rare term outside it (tiny, huge, denormal, inf, nan) is parked in a small LDS
+// queue and added to the stored slab with fp32 atomics afterwards; if the queue overflows -- a first trip
+// that says nothing about the rest -- the workgroup starts over with the fp32 LDS atomics.
+constexpr int QCAP = 512;
+struct FixedQueue {
+    int count;
+    int cell[QCAP];
+    float val[QCAP];
+};
+
+__device__ __forceinline__ bool make_window(uint32_t maxbits, int margin, int span, int &e_lo)
+{
+    const int e = (int)(maxbits >> 23);               // biased exponent of the largest |term|
+    if (e == 0 || e + margin >= 255) return false;    // only zeros and denormals, or inf / nan among them
+    e_lo = e + margin - span + 1;
+    if (e_lo < 1) e_lo = 1;
+    return true;
+}
+
+// Adds t to the cell if it lies in the window; returns true when the caller has to queue it.
+__device__ __forceinline__ bool fixed_add(unsigned long long *cell, float t, int e_lo, int span)
+{
+    const uint32_t b = __float_as_uint(t);
+    const uint32_t sh = ((b >> 23) & 0xffu) - (uint32_t)e_lo;
+    if (sh < (uint32_t)span) {
+        const unsigned long long mag = (unsigned long long)((b & 0x7fffffu) | 0x800000u) << sh;
+#ifdef MAM_EXP_NOATOMIC
+        if (mag == 12345ull)
+#endif
+        __hip_atomic_fetch_add(cell, (b >> 31) ? 0ull - mag : mag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return false;
+    }
+    return (b << 1) != 0u;
+}
+
+__device__ __forceinline__ void queue_push(FixedQueue &q, int cell, float t)
+{
+    const int slot = __hip_atomic_fetch_add(&q.count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (slot < QCAP) {
+        q.cell[slot] = cell;
+        q.val[slot] = t;
+    }
+}
+
+__device__ __forceinline__ float cell_value(unsigned long long c, int e_lo)
+{
+    return ldexpf((float)(long long)c, e_lo - 150);
+}
+
+__device__ __forceinline__ uint32_t magnitude_bits(float t) { return __float_as_uint(t) & 0x7fffffffu; }
+
+// Largest value over the workgroup; *slot is zero on entry (and a barrier has passed since).
+__device__ __forceinline__ uint32_t workgroup_max(uint32_t v, uint32_t *slot)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)v, o);
+        v = v > other ? v : other;
+    }
+    if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_max(slot, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __syncthreads();
+    return *slot;
+}
+
 template <int LAYOUT>
 __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
     const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
-    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int K, int M, int kc, int planes)
+    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int K, int M, int kc, int planes,
+    int span)
 {
     // planes > 1 (the module's `splits`): argmax / argmin are [plane][N*M] arrays of absolute k, one pair
     // per K range, w_sel (if any) [plane][2][N*M]; every plane scatters the same grad
-    extern __shared__ float hist[];
+    extern __shared__ unsigned long long cells[];      // kc cells; the fp32 fallback uses the same bytes
+    __shared__ FixedQueue q;
+    __shared__ uint32_t s_max;
+    float *hist = reinterpret_cast<float *>(cells);
     const int n = blockIdx.x;
     const int tid = threadIdx.x;
     const float *g_row = grad + (int64_t)n * M;
-    for (int k0 = 0; k0 < K; k0 += kc) {
-        const int kn = (K - k0) < kc ? (K - k0) : kc;
-        for (int i = tid; i < kn; i += NT_X) hist[i] = 0.0f;
-        __syncthreads();
-        for (int pl = 0; pl < planes; ++pl) {
+
+    // one trip: four outputs per thread; all index loads, then all weight gathers, so that the gather
+    // latencies overlap instead of adding up
+    float g[4], wv1[4], wv2[4];
+    int a1[4], a2[4];
+    auto load_trip = [&](int pl, int mb, int k0, int kn) {
         const int32_t *amax_row = argmax + pl * nm + (int64_t)n * M;
         const int32_t *amin_row = argmin + pl * nm + (int64_t)n * M;
         const float *w_sel_pl = w_sel ? w_sel + pl * 2 * nm : nullptr;
-        // four outputs per thread and trip: all index loads, then all weight gathers, then the
-        // LDS adds, so that the gather latencies overlap instead of adding up
-        for (int mb = tid; mb < M; mb += 4 * NT_X) {
-            float g[4], wv1[4], wv2[4];
-            int a1[4], a2[4];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int m = mb + u * NT_X;
+        for (int u = 0; u < 4; ++u) {
+            const int m = mb + u * NT_X;
+            const bool ok = m < M;
+            g[u] = ok ? g_row[m] : 0.0f;
+            a1[u] = ok ? amax_row[m] - k0 : -1;
+            a2[u] = ok ? amin_row[m] - k0 : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int m = mb + u * NT_X;
+            // the forward can hand over the selected weights; otherwise gather them
+            if (w_sel_pl) {
                 const bool ok = m < M;
-                g[u] = ok ? g_row[m] : 0.0f;
-                a1[u] = ok ? amax_row[m] - k0 : -1;
-                a2[u] = ok ? amin_row[m] - k0 : -1;
+                wv1[u] = ok ? w_sel_pl[(int64_t)n * M + m] : 0.0f;
+                wv2[u] = ok ? w_sel_pl[nm + (int64_t)n * M + m] : 0.0f;
+            } else {
+                wv1[u] = (unsigned)a1[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a1[u] + k0, m) : 0.0f;
+                wv2[u] = (unsigned)a2[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a2[u] + k0, m) : 0.0f;
             }
+        }
+    };
+
+    if (tid == 0) {
+        s_max = 0u;
+        q.count = 0;
+    }
+    __syncthreads();
+    bool fixed = span >= 8;
+    bool loaded = false;       // the first trip of chunk 0 is in the registers
+    int e_lo = 1;
+    if (fixed) {
+        const int kn0 = K < kc ? K : kc;
+        load_trip(0, tid, 0, kn0);
+        loaded = true;
+        uint32_t mx = 0u;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int m = mb + u * NT_X;
-                // the forward can hand over the selected weights; otherwise gather them
-                if (w_sel_pl) {
-                    const bool ok = m < M;
-                    wv1[u] = ok ? w_sel_pl[(int64_t)n * M + m] : 0.0f;
-                    wv2[u] = ok ? w_sel_pl[nm + (int64_t)n * M + m] : 0.0f;
-                } else {
-                    wv1[u] = (unsigned)a1[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a1[u] + k0, m) : 0.0f;
-                    wv2[u] = (unsigned)a2[u] < (unsigned)kn ? load_w<LAYOUT>(w, ldw, a2[u] + k0, m) : 0.0f;
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t b1 = magnitude_bits(wv1[u] * g[u]), b2 = magnitude_bits(wv2[u] * g[u]);
+            mx = mx > b1 ? mx : b1;
+            mx = mx > b2 ? mx : b2;
+        }
+        const bool whole_row = planes == 1 && M <= 4 * NT_X && K <= kc;
+        fixed = make_window(workgroup_max(mx, &s_max), whole_row ? 0 : 4, span, e_lo);
+    }
+    for (int k0 = 0; k0 < K; k0 += kc) {
+        const int kn = (K - k0) < kc ? (K - k0) : kc;
+        for (int attempt = fixed ? 0 : 1; attempt < 2; ++attempt) {
+            const bool fx = attempt == 0;
+            if (fx) for (int i = tid; i < kn; i += NT_X) cells[i] = 0ull;
+            else for (int i = tid; i < kn; i += NT_X) hist[i] = 0.0f;
+            __syncthreads();
+            for (int pl = 0; pl < planes; ++pl) {
+                for (int mb = tid; mb < M; mb += 4 * NT_X) {
+                    if (!loaded) load_trip(pl, mb, k0, kn);
+                    loaded = false;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if ((unsigned)a1[u] < (unsigned)kn) {
+                            const float t = wv1[u] * g[u];
+                            if (!fx) lds_add(&hist[a1[u]], t);
+                            else if (fixed_add(&cells[a1[u]], t, e_lo, span)) queue_push(q, k0 + a1[u], t);
+                        }
+                        if ((unsigned)a2[u] < (unsigned)kn) {
+                            const float t = wv2[u] * g[u];
+                            if (!fx) lds_add(&hist[a2[u]], t);
+                            else if (fixed_add(&cells[a2[u]], t, e_lo, span)) queue_push(q, k0 + a2[u], t);
+                        }
+                    }
                 }
             }
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if ((unsigned)a1[u] < (unsigned)kn) lds_add(&hist[a1[u]], wv1[u] * g[u]);
-                if ((unsigned)a2[u] < (unsigned)kn) lds_add(&hist[a2[u]], wv2[u] * g[u]);
+            __syncthreads();
+            const int queued = fx ? q.count : 0;
+            __syncthreads();
+            if (queued > QCAP) {       // the window was a bad guess: this chunk and the rest with fp32 atomics
+                if (tid == 0) q.count = 0;
+                fixed = false;
+                continue;
             }
+            float *dst = x_grad + (int64_t)n * K;
+            if (fx) for (int i = tid; i < kn; i += NT_X) dst[k0 + i] = cell_value(cells[i], e_lo);
+            else for (int i = tid; i < kn; i += NT_X) dst[k0 + i] = hist[i];
+            if (queued > 0) {
+                __threadfence();
+                __syncthreads();
+                for (int i = tid; i < queued; i += NT_X)
+                    __hip_atomic_fetch_add(&dst[q.cell[i]], q.val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                if (tid == 0) q.count = 0;
+            }
+            __syncthreads();
+            break;
         }
-        }
-        __syncthreads();
-        float *dst = x_grad + (int64_t)n * K + k0;
-        for (int i = tid; i < kn; i += NT_X) dst[i] = hist[i];
-        __syncthreads();
     }
 }
 
-// x_grad for large batches: a workgroup owns R = 4 .. 16 batch rows with their whole K cells in LDS,
+// x_grad for large batches: a workgroup owns R = 2 .. 16 batch rows with their whole K cells in LDS,
 // and the lanes of a wave are spread over those rows (64 / R lanes per row, 4 consecutive neurons
 // each).  The selections of ONE batch row pile up on the few k where |x| is largest, so in
 // mam_bwd_x_kernel most lanes of an instruction meet a contender; here only the 64 / R lanes of the
-// same row can, a compare-and-swap round settles nearly all of them, and the loads of a wave are
-// whole 64-byte (R = 16) to 256-byte (R = 4) pieces of R rows.
+// same row can, and the loads of a wave are whole 64-byte (R = 16) to 512-byte (R = 2) pieces of R rows.
+// Cells are 64-bit fixed point as above; the fp32 fallback settles a term by one compare-and-swap round
+// where it can.
 template <int LAYOUT>
 __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
     const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
     const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int N, int K, int M, int log2r,
-    int planes)
+    int planes, int span)
 {
-    extern __shared__ float hist[];   // [R][K]
+    extern __shared__ unsigned long long cells[];   // [R][K]
+    __shared__ FixedQueue q;
+    __shared__ uint32_t s_max;
+    float *hist = reinterpret_cast<float *>(cells);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int R = 1 << log2r;
     const int lpr = 64 >> log2r;                  // lanes per batch row
@@ -130,60 +266,106 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
     const int n = blockIdx.x * R + r;
     const bool row_ok = n < N;
     const int m_step = (NT_W / 64) * lpr * 4;     // neurons of a row the workgroup covers per trip
-    for (int i = tid; i < R * K; i += NT_W) hist[i] = 0.0f;
-    __syncthreads();
+    const int trips = (M + m_step - 1) / m_step;     // the same for every thread: lanes past M hold no item
 
     float4 g = make_float4(0.f, 0.f, 0.f, 0.f), s1 = g, s2 = g;
-    int4 i1, i2;
-    float *row = hist + r * K;
-    const int trips = (M + m_step - 1) / m_step;     // the same for every thread: lanes past M hold no item
-    for (int pl = 0; pl < planes; ++pl) {            // one (argmax, argmin) pair per K range
-    const int32_t *amax_pl = argmax + pl * nm, *amin_pl = argmin + pl * nm;
-    const float *w_sel_pl = w_sel ? w_sel + pl * 2 * nm : nullptr;
-    auto load = [&](int m) {
-        if (row_ok && m < M) {
-            const int64_t o = (int64_t)n * M + m;
-            g = *reinterpret_cast<const float4 *>(grad + o);
-            i1 = *reinterpret_cast<const int4 *>(amax_pl + o);
-            i2 = *reinterpret_cast<const int4 *>(amin_pl + o);
-            if (w_sel_pl) {
-                s1 = *reinterpret_cast<const float4 *>(w_sel_pl + o);
-                s2 = *reinterpret_cast<const float4 *>(w_sel_pl + nm + o);
-            }
-        } else {
-            i1 = make_int4(-1, -1, -1, -1);
-            i2 = i1;
-        }
-    };
-    int m = (wave * lpr + j) * 4;
-    load(m);
-    for (int t = 0; t < trips; ++t) {
-        const float4 cg = g, c1 = s1, c2 = s2;
-        const int4 a1 = i1, a2 = i2;
-        const int mc = m;
-        m += m_step;
-        load(m);         // the next trip's loads are in flight while this one is scattered
-        const float gv[4] = {cg.x, cg.y, cg.z, cg.w};
-        const int k1[4] = {a1.x, a1.y, a1.z, a1.w}, k2[4] = {a2.x, a2.y, a2.z, a2.w};
-        float w1[4] = {c1.x, c1.y, c1.z, c1.w}, w2[4] = {c2.x, c2.y, c2.z, c2.w};
-        if (!w_sel) {
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                w1[u] = (unsigned)k1[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k1[u], mc + u) : 0.0f;
-                w2[u] = (unsigned)k2[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k2[u], mc + u) : 0.0f;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            if ((unsigned)k1[u] < (unsigned)K) lds_add_sparse(&row[k1[u]], w1[u] * gv[u]);
-            if ((unsigned)k2[u] < (unsigned)K) lds_add_sparse(&row[k2[u]], w2[u] * gv[u]);
-        }
-    }
+    int4 i1 = make_int4(-1, -1, -1, -1), i2 = i1;
+// (a macro, not a lambda: captured by reference the five vectors end up in scratch memory)
+#define MAM_LOAD_ITEM(pl, m)                                                                        \
+    do {                                                                                            \
+        if (row_ok && (m) < M) {                                                                    \
+            const int64_t o_ = (int64_t)n * M + (m);                                                \
+            g = *reinterpret_cast<const float4 *>(grad + o_);                                       \
+            i1 = *reinterpret_cast<const int4 *>(argmax + (pl) * nm + o_);                          \
+            i2 = *reinterpret_cast<const int4 *>(argmin + (pl) * nm + o_);                          \
+            if (w_sel) {                                                                            \
+                s1 = *reinterpret_cast<const float4 *>(w_sel + (pl) * 2 * nm + o_);                 \
+                s2 = *reinterpret_cast<const float4 *>(w_sel + (pl) * 2 * nm + nm + o_);            \
+            }                                                                                       \
+        } else {                                                                                    \
+            i1 = make_int4(-1, -1, -1, -1);                                                         \
+            i2 = i1;                                                                                \
+        }                                                                                           \
+    } while (0)
+    const int m_first = (wave * lpr + j) * 4;
+
+    if (tid == 0) {
+        s_max = 0u;
+        q.count = 0;
     }
     __syncthreads();
+    bool fixed = span >= 8 && w_sel != nullptr;    // (a window needs the terms of the first trip: handed-over weights)
+    int e_lo = 1;
+    if (fixed) {
+        MAM_LOAD_ITEM(0, m_first);
+        uint32_t mx = 0u;
+        if (row_ok && m_first < M) {
+            const float t[8] = {s1.x * g.x, s1.y * g.y, s1.z * g.z, s1.w * g.w, s2.x * g.x, s2.y * g.y, s2.z * g.z, s2.w * g.w};
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t b = magnitude_bits(t[u]);
+                mx = mx > b ? mx : b;
+            }
+        }
+        fixed = make_window(workgroup_max(mx, &s_max), 4, span, e_lo);
+    }
     const int rows = (N - blockIdx.x * R) < R ? (N - blockIdx.x * R) : R;
     float *dst = x_grad + (int64_t)blockIdx.x * R * K;
-    for (int i = tid; i < rows * K; i += NT_W) dst[i] = hist[i];
+    for (int attempt = fixed ? 0 : 1; attempt < 2; ++attempt) {
+        const bool fx = attempt == 0;
+        if (fx) for (int i = tid; i < R * K; i += NT_W) cells[i] = 0ull;
+        else for (int i = tid; i < R * K; i += NT_W) hist[i] = 0.0f;
+        __syncthreads();
+        for (int pl = 0; pl < planes; ++pl) {            // one (argmax, argmin) pair per K range
+            int m = m_first;
+            MAM_LOAD_ITEM(pl, m);
+            for (int t = 0; t < trips; ++t) {
+                const float4 cg = g, c1 = s1, c2 = s2;
+                const int4 a1 = i1, a2 = i2;
+                const int mc = m;
+                m += m_step;
+                MAM_LOAD_ITEM(pl, m);         // the next trip's loads are in flight while this one is scattered
+                const float gv[4] = {cg.x, cg.y, cg.z, cg.w};
+                const int k1[4] = {a1.x, a1.y, a1.z, a1.w}, k2[4] = {a2.x, a2.y, a2.z, a2.w};
+                float w1[4] = {c1.x, c1.y, c1.z, c1.w}, w2[4] = {c2.x, c2.y, c2.z, c2.w};
+                if (!w_sel) {
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        w1[u] = (unsigned)k1[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k1[u], mc + u) : 0.0f;
+                        w2[u] = (unsigned)k2[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k2[u], mc + u) : 0.0f;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if ((unsigned)k1[u] < (unsigned)K) {
+                        const float tv = w1[u] * gv[u];
+                        if (!fx) lds_add_sparse(&hist[r * K + k1[u]], tv);
+                        else if (fixed_add(&cells[r * K + k1[u]], tv, e_lo, span)) queue_push(q, r * K + k1[u], tv);
+                    }
+                    if ((unsigned)k2[u] < (unsigned)K) {
+                        const float tv = w2[u] * gv[u];
+                        if (!fx) lds_add_sparse(&hist[r * K + k2[u]], tv);
+                        else if (fixed_add(&cells[r * K + k2[u]], tv, e_lo, span)) queue_push(q, r * K + k2[u], tv);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const int queued = fx ? q.count : 0;
+        __syncthreads();
+        if (queued > QCAP) continue;      // the window was a bad guess: once more with fp32 atomics
+        if (fx) for (int i = tid; i < rows * K; i += NT_W) dst[i] = cell_value(cells[i], e_lo);
+        else for (int i = tid; i < rows * K; i += NT_W) dst[i] = hist[i];
+        if (queued > 0) {
+            __threadfence();
+            __syncthreads();
+            for (int i = tid; i < queued; i += NT_W)
+                if (q.cell[i] < rows * K)
+                    __hip_atomic_fetch_add(&dst[q.cell[i]], q.val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        break;
+    }
+#undef MAM_LOAD_ITEM
 }
 
 // Scatter of one (batch row, 4 consecutive neurons) item into the slab histogram.
@@ -409,6 +591,10 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
 // 64 KiB the kernel attribute has to be raised first, once per device, which the device's set-up does
 // for every kernel of this file.
 static int g_lds_floats[kMaxDevices];
+#ifndef MAM_BWD_ROWS_LDS
+#define MAM_BWD_ROWS_LDS (64 * 1024)
+#endif
+constexpr int64_t kRowsLdsBytes = MAM_BWD_ROWS_LDS;
 
 static int setup_device(int dev)
 {
@@ -442,24 +628,28 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
     if (dev < 0) return dev;
     const int lds_cap = g_lds_floats[dev];
     const int cus = num_cus();
+    // 64-bit fixed-point cells: room for 2 * M * planes terms of 24 + span - 1 bits each, and one bit to spare
+    int count_bits = 1;
+    while (((int64_t)1 << count_bits) <= 2 * M * planes) ++count_bits;
+    const int span = 63 - 24 - count_bits;
     const bool x_rows = N >= 2048 && K * 16 <= 64 * 1024 && (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
                         ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) &&
                         ((uintptr_t)w_sel % 16 == 0);
     if (x_grad && x_rows) {
-        // as many rows per workgroup (4, 8 or 16) as fit 64 KiB of LDS
-        int log2r = 2;
-        while (log2r < 4 && ((int64_t)2 << log2r) * K * 4 <= 64 * 1024) ++log2r;
+        // as many rows per workgroup (2 to 16) as fit 64 KiB of LDS in 8-byte cells
+        int log2r = 1;
+        while (log2r < 4 && ((int64_t)2 << log2r) * K * 8 <= kRowsLdsBytes) ++log2r;
         const int R = 1 << log2r;
         hipLaunchKernelGGL((mam_bwd_x_rows_kernel<LAYOUT>), dim3((unsigned)ceil_div(N, R)), dim3(NT_W),
-                           (size_t)R * K * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M, x_grad,
-                           (int)N, (int)K, (int)M, log2r, planes);
+                           (size_t)R * K * 8, st, w, ldw, grad, argmax, argmin, w_sel, N * M, x_grad,
+                           (int)N, (int)K, (int)M, log2r, planes, span);
         rc = check_launch("mam_bwd_x_rows_kernel");
         if (rc != MAM_OK) return rc;
     } else if (x_grad) {
-        const int kc = (int)(K < lds_cap ? K : lds_cap);
+        const int kc = (int)(K < lds_cap / 2 ? K : lds_cap / 2);
         hipLaunchKernelGGL((mam_bwd_x_kernel<LAYOUT>), dim3((unsigned)N), dim3(NT_X),
-                           (size_t)kc * sizeof(float), st, w, ldw, grad, argmax, argmin, w_sel, N * M,
-                           x_grad, (int)K, (int)M, kc, planes);
+                           (size_t)kc * 8, st, w, ldw, grad, argmax, argmin, w_sel, N * M,
+                           x_grad, (int)K, (int)M, kc, planes, span);
         rc = check_launch("mam_bwd_x_kernel");
         if (rc != MAM_OK) return rc;
     }
@@ -528,10 +718,12 @@ int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t
 {
     const int dev = ensure_device();
     if (dev < 0) return dev;
-    const int kc = (int)(K < g_lds_floats[dev] ? K : g_lds_floats[dev]);
-    hipLaunchKernelGGL((mam_bwd_x_kernel<MAM_W_MK>), dim3((unsigned)N), dim3(NT_X), (size_t)kc * sizeof(float),
+    const int kc = (int)(K < g_lds_floats[dev] / 2 ? K : g_lds_floats[dev] / 2);
+    int count_bits = 1;
+    while (((int64_t)1 << count_bits) <= 2 * M) ++count_bits;
+    hipLaunchKernelGGL((mam_bwd_x_kernel<MAM_W_MK>), dim3((unsigned)N), dim3(NT_X), (size_t)kc * 8,
                        st, (const float *)nullptr, (int64_t)0, grad, argmax, argmin, w_sel, N * M, x_grad, (int)K,
-                       (int)M, kc, 1);
+                       (int)M, kc, 1, 63 - 24 - count_bits);
     return check_launch("mam_bwd_x_kernel");
 }
 

@@ -118,12 +118,14 @@ __device__ __forceinline__ void resolve(const Params &p, int n, int m, int kb, i
 // A zero extreme carries the sign of the FIRST zero product; the hardware max/min may have
 // kept another zero's sign.  Rare (whole column of products has no positive / no negative
 // entry), so a plain scan is enough.
+// (Not inlined, and handed plain pointers: a reference to the kernel's parameter block would force a
+// copy of the block into every lane's scratch memory.)
 template <int LAYOUT>
-__device__ __noinline__ float first_zero_product(const Params &p, int n, int m, int kbegin, int kend)
+__device__ __noinline__ float first_zero_product(const float *xr, const float *w, int64_t ldw, int m, int kbegin,
+                                                 int kend)
 {
-    const float *xr = p.x + (int64_t)n * p.ldx;
     for (int k = kbegin; k < kend; ++k) {
-        const float prod = xr[k] * load_w<LAYOUT>(p.w, p.ldw, k, m);
+        const float prod = xr[k] * load_w<LAYOUT>(w, ldw, k, m);
         if (prod == 0.0f) return prod;
     }
     return 0.0f;
@@ -140,8 +142,8 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
         resolve<LAYOUT>(p, n, m, gmax * G, p.K - 1, vmax, hi, ih, wh, xh);
         resolve<LAYOUT>(p, n, m, gmin * G, p.K - 1, vmin, lo, il, wl, xl);
     } else {
-        if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m, 0, p.K);
-        if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m, 0, p.K);
+        if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p.x + (int64_t)n * p.ldx, p.w, p.ldw, m, 0, p.K);
+        if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p.x + (int64_t)n * p.ldx, p.w, p.ldw, m, 0, p.K);
     }
     float s = hi + lo;
     if (p.bias) s = s + p.bias[m];
@@ -760,8 +762,8 @@ __global__ __launch_bounds__(256) void mam_fwd_range_sum_kernel(const Params p)
             p.argmax[(int64_t)s * nm + o] = ih;
             p.argmin[(int64_t)s * nm + o] = il;
         } else {
-            if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p, n, m, kb, ke);
-            if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p, n, m, kb, ke);
+            if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p.x + (int64_t)n * p.ldx, p.w, p.ldw, m, kb, ke);
+            if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p.x + (int64_t)n * p.ldx, p.w, p.ldw, m, kb, ke);
         }
         const float v = hi + lo;
         total = s == 0 ? v : total + v;

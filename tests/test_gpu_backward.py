@@ -235,3 +235,82 @@ def test_x_grad_on_the_second_stream_or_not(fork):
             assert abs(sums - (xo.astype(np.float64).sum() + wo.astype(np.float64).sum())) < 1e-2
     finally:
         capi.set_option(capi.OPT_BACKWARD_FORK, capi.BACKWARD_FORK_AUTO)
+
+
+def _dynamic_range_grad(N, M, pattern, seed):
+    """grad whose terms span far more binades than a 64-bit fixed-point window holds."""
+    g = torch.Generator().manual_seed(seed)
+    grad = torch.randn(N, M, generator=g)
+    if pattern == "few tiny":            # a handful of terms 2^-70 below the rest: parked and added afterwards
+        idx = torch.randint(0, M, (N, 3), generator=g)
+        grad.scatter_(1, idx, torch.full((N, 3), 2.0 ** -70))
+    elif pattern == "few huge":          # a few terms 2^40 above the first ones
+        idx = torch.randint(M // 2, M, (N, 2), generator=g)
+        grad.scatter_(1, idx, torch.full((N, 2), 2.0 ** 40))
+    elif pattern == "head huge":         # the first neurons decide the window, everything after them is below it
+        grad[:, 4:] *= 2.0 ** -60
+    elif pattern == "head tiny":         # ... or far above it
+        grad[:, :M // 2] *= 2.0 ** -60
+    elif pattern == "every binade":      # exponents spread over 100 binades
+        grad *= torch.exp2(torch.randint(-60, 40, (N, M), generator=g).float())
+    elif pattern == "denormal":
+        grad *= 2.0 ** -140
+    return grad
+
+
+@pytest.mark.parametrize("pattern", ["few tiny", "few huge", "head huge", "head tiny", "every binade", "denormal"])
+@pytest.mark.parametrize("shape", [(40, 256, 4100), (2048, 128, 520)])
+def test_x_grad_over_a_wide_dynamic_range(shape, pattern):
+    """x_grad accumulates in 64-bit fixed point inside a window of exponents; terms outside the window take
+    the fp32 path, and a window that fits almost nothing makes the workgroup start over with fp32 atomics.
+    Every one of those routes has to meet the same bar, for the one-row-per-workgroup kernel (first shape)
+    and the rows-per-workgroup kernel of large batches (second shape)."""
+    N, K, M = shape
+    x, w, _ = random_case(N, K, M, seed=N + M)
+    grad = _dynamic_range_grad(N, M, pattern, seed=K)
+    _, amax, amin = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+    _check(x, w, grad, amax, amin, "%s %s" % (pattern, shape,), layouts=(1,))
+
+
+@pytest.mark.parametrize("shape", [(40, 256, 4100), (2048, 128, 520)])
+def test_x_grad_with_non_finite_terms(shape):
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    N, K, M = shape
+    x, w, grad = random_case(N, K, M, seed=N)
+    grad[1, 5], grad[2, 7], grad[3, 9] = float("inf"), float("nan"), float("-inf")
+    c, amax, amin = capi.fc_forward(x.to(dev), w.to(dev), capi.W_MK)
+    a1, a2 = amax.cpu().numpy(), amin.cpu().numpy()
+    cols = torch.arange(M)[None, :]
+    w_sel = torch.stack([w[cols, amax.cpu().long()], w[cols, amin.cpu().long()]]).contiguous().to(dev)
+    xg, _ = capi.fc_backward(x.to(dev), w.to(dev), grad.to(dev), amax, amin, capi.W_MK, want_w=False, w_sel=w_sel)
+    torch.cuda.synchronize()
+    xo, _ = oracle.backward(x.numpy(), w.numpy(), grad.numpy(), a1, a2, oracle.W_MK)
+    got = xg.cpu().numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(xo))
+    assert np.array_equal(np.isinf(got), np.isinf(xo)) and np.array_equal(got[np.isinf(xo)], xo[np.isinf(xo)])
+    fin = np.isfinite(xo)
+    np.testing.assert_allclose(got[fin], xo[fin], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(256, 512, 1024), (4096, 256, 512)])
+def test_x_grad_is_reproducible_bit_for_bit(shape):
+    """Inside the window the sum of a cell is exact, so neither the order in which lanes arrive nor the
+    launch changes a bit of x_grad."""
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    N, K, M = shape
+    x, w, grad = random_case(N, K, M, seed=3)
+    xd, wd, gd = x.to(dev), w.to(dev), grad.to(dev)
+    ws = torch.empty(2, N, M, device=dev)
+    xs = torch.empty(2, N, M, device=dev)
+    c, amax, amin = capi.fc_forward(xd, wd, capi.W_MK, w_sel=ws, x_sel=xs)
+    first, _ = capi.fc_backward(xd, wd, gd, amax, amin, capi.W_MK, want_w=False, w_sel=ws)
+    for _ in range(3):
+        again, _ = capi.fc_backward(xd, wd, gd, amax, amin, capi.W_MK, want_w=False, w_sel=ws)
+        assert torch.equal(first, again)
+    # and it is the correctly rounded exact sum: fp64 accumulation of the fp32 terms, rounded once
+    xo, _ = oracle.backward(x.numpy(), w.numpy(), grad.numpy(), amax.cpu().numpy(), amin.cpu().numpy(), oracle.W_MK)
+    np.testing.assert_array_equal(first.cpu().numpy(), xo.astype(np.float32))
