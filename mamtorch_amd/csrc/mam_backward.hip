@@ -5,19 +5,21 @@
 // Both outputs are dense matrices that are almost entirely zero (at most 2*N*M non-zeros), so
 // the work is bandwidth: write every output byte exactly once and read the (grad, argmax, argmin)
 // triples as few times as possible.  Each workgroup OWNS a slab of an output, accumulates the
-// scattered terms for that slab in an LDS histogram with ds_add_f32, and then streams the slab to
-// HBM with coalesced stores -- no zero-fill pass and no global atomics:
+// scattered terms for that slab in LDS, and then streams the slab to HBM with coalesced stores --
+// no zero-fill pass and no global atomics:
 //
-//   x_grad : one workgroup per batch row n; histogram over k (chunked when K floats exceed LDS).
-//            From 2048 batch rows on: 4 to 16 rows per workgroup, the lanes of a wave spread over them.
-//   w_grad : one workgroup per R consecutive output neurons x KC consecutive k.  For the (M,K)
+//   x_grad : one workgroup per batch row n; cells over k (chunked when they exceed LDS).  From 2048
+//            batch rows on: 2 to 16 rows per workgroup, the lanes of a wave spread over them.  The cells
+//            are 64-bit fixed point (integer LDS atomics, exact sums, see below).
+//   w_grad : one workgroup per R consecutive output neurons x KC consecutive k, fp32 cells.  For the (M,K)
 //            layout R = 4 so a slab is 4 whole rows of the weight gradient (64 KiB: two
 //            workgroups per CU); for the (K,M) layout R = 32 so that every stored row segment is
 //            128 bytes.  From 2048 batch rows on, (M,K): up to 16 neurons per slab and the batch shared
 //            by several workgroups per slab, which add their shares to the cleared w_grad.
 //
-// Each term is one fp32 product (operand of the reference's atomicAdd); only the order of the
-// fp32 additions differs from the reference, which is itself unordered.
+// Each term is one fp32 product (operand of the reference's atomicAdd).  x_grad is the exact sum of its
+// terms rounded once; in w_grad only the order of the fp32 additions differs from the reference, which is
+// itself unordered.
 #include "mam_common.h"
 
 namespace mam {
@@ -27,9 +29,8 @@ constexpr int NT_X = 1024;
 constexpr int NT_W = 512;
 
 // ds_add_f32 costs ~3 cycles per active lane on this chip, ~190 per full 64-lane instruction,
-// whatever the addresses (an integer LDS atomic: ~5 per instruction).  x_grad keeps it: 2 to 3
-// lanes of an instruction share a key on average, so a compare-and-swap round would leave most
-// lanes to it anyway, and merging equal keys across the wave first was measured to save 10 %.
+// whatever the addresses (an integer LDS atomic: ~5 per instruction, ~8 for 64 bits).  Only the fp32
+// fallback of x_grad still uses it.
 __device__ __forceinline__ void lds_add(float *addr, float v)
 {
     __hip_atomic_fetch_add(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
