@@ -346,18 +346,19 @@ def run_sparse(torch, capi, lib, dev, args):
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     wsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)   # selected values, forward -> backward
     psel = torch.empty((2, N, M), dtype=torch.int32, device=dev)     # their positions in col/val
+    xsel = torch.empty((2, N, M), dtype=torch.float32, device=dev)   # the selected inputs
     stream = torch.cuda.current_stream(dev)
     sp = ctypes.c_void_p(stream.cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
 
     def forward():
         rc = lib.mam_csr_fc_forward(P(xd), K, P(crow), P(col), P(val), None, P(c), P(amax), P(amin), P(wsel),
-                                    P(psel), N, K, M, nnz, P(ws), ws_bytes, sp)
+                                    P(psel), P(xsel), N, K, M, nnz, P(ws), ws_bytes, sp)
         assert rc == 0, lib.mam_last_error()
 
     def backward():
         rc = lib.mam_csr_fc_backward(P(xd), K, P(crow), P(col), P(val), P(gd), P(amax), P(amin), P(wsel),
-                                     P(psel), P(xg), P(vg), N, K, M, nnz, sp)
+                                     P(psel), P(xsel), P(xg), P(vg), N, K, M, nnz, sp)
         assert rc == 0, lib.mam_last_error()
 
     # one plain 64 MiB copy kernel: the known-size reference that scales the profiler's FETCH_SIZE /
@@ -367,8 +368,8 @@ def run_sparse(torch, capi, lib, dev, args):
     del calibration_src, calibration_copy
     ms_step, ph = time_phases(torch, stream, [("forward", forward), ("backward", backward)], args.steps, args.warmup)
     triples = nnz * N                                    # stored products only
-    fwd_bytes = 12 * nnz + 4 * N * K + 12 * N * M + 16 * N * M       # + hand-over arrays
-    bwd_bytes = 4 * N * K + 12 * N * M + 16 * N * M + 4 * N * K + 4 * nnz
+    fwd_bytes = 12 * nnz + 4 * N * K + 12 * N * M + 24 * N * M       # + hand-over arrays
+    bwd_bytes = 12 * N * M + 24 * N * M + 4 * N * K + 4 * nnz
     out = {
         "config": {"workload": "Pruned CSR-sparse MAM FullyConnected fp32: 4096x4096 weight, %.0f %% of entries kept "
                                "(seeded random columns per row), W~N(0,0.02), batch 256, x~N(0,1); sparse forward + "

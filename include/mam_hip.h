@@ -204,12 +204,14 @@ int mam_selection_count(const int32_t *argmax, const int32_t *argmin, int32_t *m
  * `w_sel` and `pos_sel` (optional, may be NULL): (2, N, M) fp32 / int32 contiguous; receive, for the
  * argmax in plane 0 and the argmin in plane 1, the selected stored value and its position in
  * col/val (0.0f and -1 where an implicit zero was selected).  Handing both to mam_csr_fc_backward
- * spares that call a binary search per selection and all atomics in global memory.
+ * spares that call a binary search per selection and all atomics in global memory.  `x_sel` (optional):
+ * (2, N, M) fp32, the selected inputs x[n, argmax] / x[n, argmin] (0.0f where an implicit zero was
+ * selected); handed to mam_csr_fc_backward it spares val_grad 2 * N * M single-word gathers from x.
  */
 size_t mam_csr_fc_forward_workspace(int64_t N, int64_t K, int64_t M);
 int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                        const float *val, const float *bias, float *c, int32_t *argmax,
-                       int32_t *argmin, float *w_sel, int32_t *pos_sel, int64_t N, int64_t K,
+                       int32_t *argmin, float *w_sel, int32_t *pos_sel, float *x_sel, int64_t N, int64_t K,
                        int64_t M, int64_t nnz, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
@@ -227,13 +229,14 @@ int mam_csr_validate(const int64_t *crow, const int64_t *col, int64_t M, int64_t
 /*
  * CSR-sparse MAM backward: x_grad (N,K) dense and val_grad (nnz), both fully overwritten; either may
  * be NULL to skip it.  A selected column that is not stored in its row (an implicit zero won) has no
- * weight gradient and adds nothing to x_grad.  `w_sel` / `pos_sel` (optional, both or neither) are the
- * arrays written by mam_csr_fc_forward for the same inputs.
+ * weight gradient and adds nothing to x_grad.  `w_sel` / `pos_sel` (optional, both or neither) and `x_sel`
+ * (optional, only together with the other two) are the arrays written by mam_csr_fc_forward for the same
+ * inputs.
  */
 int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                         const float *val, const float *grad, const int32_t *argmax,
                         const int32_t *argmin, const float *w_sel, const int32_t *pos_sel,
-                        float *x_grad, float *val_grad, int64_t N, int64_t K, int64_t M,
+                        const float *x_sel, float *x_grad, float *val_grad, int64_t N, int64_t K, int64_t M,
                         int64_t nnz, void *stream);
 
 /*

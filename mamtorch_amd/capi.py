@@ -78,10 +78,10 @@ def lib():
         l.mam_fc_backward_ranges.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
                                              _i64, _i64, _ptr]
         l.mam_selection_count.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr]
-        l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+        l.mam_csr_fc_forward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                          _i64, _i64, _i64, _i64, _ptr, _size, _ptr]
         l.mam_csr_fc_backward.argtypes = [_ptr, _i64, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
-                                          _ptr, _i64, _i64, _i64, _i64, _ptr]
+                                          _ptr, _ptr, _i64, _i64, _i64, _i64, _ptr]
         l.mam_blend.argtypes = [_ptr, _ptr, _ptr, ctypes.c_float, ctypes.c_float, _ptr, _i64, _i64, _ptr]
         l.mam_apply_keep.argtypes = [_ptr, _i64, _ptr, _ptr, _i64, _i64, _ptr]
         l.mam_im2col.argtypes = [_ptr, _ptr] + [_i64] * 8 + [_ptr]
@@ -223,7 +223,7 @@ def selection_count(argmax, argmin, max_count, min_count, mode=COUNT_REFERENCE):
                                      _stream(argmax)))
 
 
-def csr_fc_forward(x, crow, col, val, M, bias=None, w_sel=None, pos_sel=None):
+def csr_fc_forward(x, crow, col, val, M, bias=None, w_sel=None, pos_sel=None, x_sel=None):
     """Returns (c, argmax, argmin); fills the optional (2,N,M) hand-over arrays for the backward."""
     l = lib()
     N, K = x.shape
@@ -234,7 +234,7 @@ def csr_fc_forward(x, crow, col, val, M, bias=None, w_sel=None, pos_sel=None):
     ws = torch.empty(max(need, 1), dtype=torch.uint8, device=x.device)
     with torch.cuda.device(x.device):
         _check(l.mam_csr_fc_forward(_p(x), _ld(x), _p(crow), _p(col), _p(val), _p(bias), _p(c), _p(amax),
-                                    _p(amin), _p(w_sel), _p(pos_sel), N, K, M, val.numel(), _p(ws), need,
+                                    _p(amin), _p(w_sel), _p(pos_sel), _p(x_sel), N, K, M, val.numel(), _p(ws), need,
                                     _stream(x)))
     return c, amax, amin
 
@@ -251,7 +251,7 @@ def csr_validate(crow, col, K):
     return int(status.item())
 
 
-def csr_fc_backward(x, crow, col, val, grad, argmax, argmin, w_sel=None, pos_sel=None):
+def csr_fc_backward(x, crow, col, val, grad, argmax, argmin, w_sel=None, pos_sel=None, x_sel=None):
     l = lib()
     N, K = x.shape
     M = crow.numel() - 1
@@ -259,7 +259,7 @@ def csr_fc_backward(x, crow, col, val, grad, argmax, argmin, w_sel=None, pos_sel
     vg = torch.empty_like(val)
     with torch.cuda.device(x.device):
         _check(l.mam_csr_fc_backward(_p(x), _ld(x), _p(crow), _p(col), _p(val), _p(grad), _p(argmax),
-                                     _p(argmin), _p(w_sel), _p(pos_sel), _p(xg), _p(vg), N, K, M, val.numel(),
+                                     _p(argmin), _p(w_sel), _p(pos_sel), _p(x_sel), _p(xg), _p(vg), N, K, M, val.numel(),
                                      _stream(x)))
     return xg, vg
 

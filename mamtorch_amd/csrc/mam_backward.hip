@@ -21,9 +21,12 @@
 // terms rounded once; in w_grad only the order of the fp32 additions differs from the reference, which is
 // itself unordered.
 #include "mam_common.h"
+#include "mam_fixed.h"
 
 namespace mam {
 namespace bwd {
+
+using namespace fixedpoint;
 
 constexpr int NT_X = 1024;
 constexpr int NT_W = 512;
@@ -48,77 +51,6 @@ __device__ __forceinline__ void lds_add_sparse(float *addr, float v)
                                                            __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                                                            __HIP_MEMORY_SCOPE_WORKGROUP);
     if (!done) lds_add(addr, v);
-}
-
-// ---- exact accumulation of x_grad in 64-bit fixed point ------------------------------------------------
-// An fp32 term is m * 2^(e - 150) with a 24-bit integer m.  Relative to a window [e_lo, e_lo + span) of
-// biased exponents it is the integer m << (e - e_lo), and integer adds are exact and commute: the cell ends
-// up with the exact sum of its terms whatever order the lanes arrive in, rounded to fp32 once when the slab
-// is stored -- and the integer LDS atomic costs ~8 cycles per 64-lane instruction where ds_add_f32 costs
-// ~190.  span leaves room for every term a cell can receive (2 * M * planes), so the sum cannot overflow.
-// The window is placed by the largest term of the workgroup's first trip (plus 4 binades where that is
-// not the whole row).  The rare term outside it (tiny, huge, denormal, inf, nan) is parked in a small LDS
-// queue and added to the stored slab with fp32 atomics afterwards; if the queue overflows -- a first trip
-// that says nothing about the rest -- the workgroup starts over with the fp32 LDS atomics.
-constexpr int QCAP = 512;
-struct FixedQueue {
-    int count;
-    int cell[QCAP];
-    float val[QCAP];
-};
-
-__device__ __forceinline__ bool make_window(uint32_t maxbits, int margin, int span, int &e_lo)
-{
-    const int e = (int)(maxbits >> 23);               // biased exponent of the largest |term|
-    if (e == 0 || e + margin >= 255) return false;    // only zeros and denormals, or inf / nan among them
-    e_lo = e + margin - span + 1;
-    if (e_lo < 1) e_lo = 1;
-    return true;
-}
-
-// Adds t to the cell if it lies in the window; returns true when the caller has to queue it.
-__device__ __forceinline__ bool fixed_add(unsigned long long *cell, float t, int e_lo, int span)
-{
-    const uint32_t b = __float_as_uint(t);
-    const uint32_t sh = ((b >> 23) & 0xffu) - (uint32_t)e_lo;
-    if (sh < (uint32_t)span) {
-        const unsigned long long mag = (unsigned long long)((b & 0x7fffffu) | 0x800000u) << sh;
-#ifdef MAM_EXP_NOATOMIC
-        if (mag == 12345ull)
-#endif
-        __hip_atomic_fetch_add(cell, (b >> 31) ? 0ull - mag : mag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        return false;
-    }
-    return (b << 1) != 0u;
-}
-
-__device__ __forceinline__ void queue_push(FixedQueue &q, int cell, float t)
-{
-    const int slot = __hip_atomic_fetch_add(&q.count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (slot < QCAP) {
-        q.cell[slot] = cell;
-        q.val[slot] = t;
-    }
-}
-
-__device__ __forceinline__ float cell_value(unsigned long long c, int e_lo)
-{
-    return ldexpf((float)(long long)c, e_lo - 150);
-}
-
-__device__ __forceinline__ uint32_t magnitude_bits(float t) { return __float_as_uint(t) & 0x7fffffffu; }
-
-// Largest value over the workgroup; *slot is zero on entry (and a barrier has passed since).
-__device__ __forceinline__ uint32_t workgroup_max(uint32_t v, uint32_t *slot)
-{
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const uint32_t other = (uint32_t)__shfl_xor((int)v, o);
-        v = v > other ? v : other;
-    }
-    if ((threadIdx.x & 63) == 0) __hip_atomic_fetch_max(slot, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    __syncthreads();
-    return *slot;
 }
 
 template <int LAYOUT>
@@ -630,9 +562,7 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
     const int lds_cap = g_lds_floats[dev];
     const int cus = num_cus();
     // 64-bit fixed-point cells: room for 2 * M * planes terms of 24 + span - 1 bits each, and one bit to spare
-    int count_bits = 1;
-    while (((int64_t)1 << count_bits) <= 2 * M * planes) ++count_bits;
-    const int span = 63 - 24 - count_bits;
+    const int span = window_span(2 * M * planes);
     const bool x_rows = N >= 2048 && K * 16 <= 64 * 1024 && (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
                         ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) &&
                         ((uintptr_t)w_sel % 16 == 0);
@@ -720,11 +650,9 @@ int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t
     const int dev = ensure_device();
     if (dev < 0) return dev;
     const int kc = (int)(K < g_lds_floats[dev] / 2 ? K : g_lds_floats[dev] / 2);
-    int count_bits = 1;
-    while (((int64_t)1 << count_bits) <= 2 * M) ++count_bits;
     hipLaunchKernelGGL((mam_bwd_x_kernel<MAM_W_MK>), dim3((unsigned)N), dim3(NT_X), (size_t)kc * 8,
                        st, (const float *)nullptr, (int64_t)0, grad, argmax, argmin, w_sel, N * M, x_grad, (int)K,
-                       (int)M, kc, 1, 63 - 24 - count_bits);
+                       (int)M, kc, 1, window_span(2 * M));
     return check_launch("mam_bwd_x_kernel");
 }
 

@@ -35,6 +35,7 @@
 // x_grad is accumulated in an LDS histogram and stored once, val_grad takes global atomic adds (at
 // most N contenders per entry).
 #include "mam_common.h"
+#include "mam_fixed.h"
 
 namespace mam {
 namespace csr {
@@ -87,7 +88,8 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
     const float *__restrict__ xT, int ldt, const int64_t *__restrict__ crow,
     const int64_t *__restrict__ col, const float *__restrict__ val, const float *__restrict__ bias,
     float *__restrict__ c, int32_t *__restrict__ argmax, int32_t *__restrict__ argmin,
-    float *__restrict__ w_sel, int32_t *__restrict__ pos_sel, int N, int K, int M, int vec_out)
+    float *__restrict__ w_sel, int32_t *__restrict__ pos_sel, float *__restrict__ x_sel, int N, int K, int M,
+    int vec_out)
 {
     typedef typename XVec<TI>::type xvec;
     constexpr int TILE_N = 64 * TI;
@@ -100,6 +102,8 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
     float (*out_wl)[TILE_N] = reinterpret_cast<float (*)[TILE_N]>(out_lds + 4 * ROWS * TILE_N);
     int (*out_ph)[TILE_N] = reinterpret_cast<int (*)[TILE_N]>(out_lds + 5 * ROWS * TILE_N);
     int (*out_pl)[TILE_N] = reinterpret_cast<int (*)[TILE_N]>(out_lds + 6 * ROWS * TILE_N);
+    float (*out_xh)[TILE_N] = reinterpret_cast<float (*)[TILE_N]>(out_lds + 7 * ROWS * TILE_N);
+    float (*out_xl)[TILE_N] = reinterpret_cast<float (*)[TILE_N]>(out_lds + 8 * ROWS * TILE_N);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -277,7 +281,7 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
         // other zero's sign, so a second entry selected for a zero extreme is recomputed (rare: a branch
         // that whole waves skip).
         int ri[2][TI];
-        float rw[2][TI];
+        float rw[2][TI], rx[2][TI];
 #pragma unroll
         for (int t = 0; t < TI; ++t) {
 #pragma unroll
@@ -299,22 +303,24 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
                     pos = e;
                     ri[ext][t] = (int)cc;
                     rw[ext][t] = w;
+                    rx[ext][t] = x_sel ? xT[cc * (int64_t)ldt + nl + t] : 0.0f;
                 } else {
                     pos = -1;
                     ri[ext][t] = -1;
                     rw[ext][t] = 0.0f;
+                    rx[ext][t] = 0.0f;
                 }
             }
         }
 
 #pragma unroll
         for (int t = 0; t < TI; ++t) {
-            float hi = vmax[t], lo = vmin[t], wh = rw[0][t], wl = rw[1][t];
+            float hi = vmax[t], lo = vmin[t], wh = rw[0][t], wl = rw[1][t], xh = rx[0][t], xl_ = rx[1][t];
             int ih = ri[0][t], il = ri[1][t], ph = pmax[t], pl = pmin[t];
             if (has_zero) {
                 const float z = lane_elem(zx, t) * 0.0f;
-                if (ih < 0 || z > hi || (z == hi && missing < ih)) { hi = z; ih = missing; wh = 0.0f; ph = -1; }
-                if (il < 0 || z < lo || (z == lo && missing < il)) { lo = z; il = missing; wl = 0.0f; pl = -1; }
+                if (ih < 0 || z > hi || (z == hi && missing < ih)) { hi = z; ih = missing; wh = 0.0f; xh = 0.0f; ph = -1; }
+                if (il < 0 || z < lo || (z == lo && missing < il)) { lo = z; il = missing; wl = 0.0f; xl_ = 0.0f; pl = -1; }
             }
             float s = hi + lo;
             if (bias) s = s + bm;
@@ -324,6 +330,8 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
             out_lo[wave][o] = il;
             out_wh[wave][o] = wh;
             out_wl[wave][o] = wl;
+            out_xh[wave][o] = xh;
+            out_xl[wave][o] = xl_;
             out_ph[wave][o] = ph < 0 ? -1 : (int)(beg + ph);
             out_pl[wave][o] = pl < 0 ? -1 : (int)(beg + pl);
         }
@@ -353,6 +361,10 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
                 *reinterpret_cast<int4 *>(pos_sel + base) = make_int4(out_ph[r0][o], out_ph[r0 + 1][o], out_ph[r0 + 2][o], out_ph[r0 + 3][o]);
                 *reinterpret_cast<int4 *>(pos_sel + nm + base) = make_int4(out_pl[r0][o], out_pl[r0 + 1][o], out_pl[r0 + 2][o], out_pl[r0 + 3][o]);
             }
+            if (x_sel) {
+                *reinterpret_cast<float4 *>(x_sel + base) = make_float4(out_xh[r0][o], out_xh[r0 + 1][o], out_xh[r0 + 2][o], out_xh[r0 + 3][o]);
+                *reinterpret_cast<float4 *>(x_sel + nm + base) = make_float4(out_xl[r0][o], out_xl[r0 + 1][o], out_xl[r0 + 2][o], out_xl[r0 + 3][o]);
+            }
         } else {
             for (int r = r0; r < r0 + 4 && m0 + r < M; ++r) {
                 const int64_t dst = (int64_t)n * M + m0 + r;
@@ -361,6 +373,7 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
                 argmin[dst] = out_lo[r][o];
                 if (w_sel) { w_sel[dst] = out_wh[r][o]; w_sel[nm + dst] = out_wl[r][o]; }
                 if (pos_sel) { pos_sel[dst] = out_ph[r][o]; pos_sel[nm + dst] = out_pl[r][o]; }
+                if (x_sel) { x_sel[dst] = out_xh[r][o]; x_sel[nm + dst] = out_xl[r][o]; }
             }
         }
     }
@@ -430,7 +443,10 @@ __device__ __forceinline__ void lds_add_sparse(float *addr, float v)
     if (!done) __hip_atomic_fetch_add(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
-constexpr int RB = 16;           // CSR rows per val_grad workgroup
+#ifndef MAM_CSR_RB
+#define MAM_CSR_RB 16
+#endif
+constexpr int RB = MAM_CSR_RB;   // CSR rows per val_grad workgroup
 constexpr int VAL_CAP = 16384;   // histogram floats per pass (64 KiB)
 
 // val_grad of the entries of RB consecutive CSR rows, from the entry positions recorded by the
@@ -438,8 +454,8 @@ constexpr int VAL_CAP = 16384;   // histogram floats per pass (64 KiB)
 __global__ __launch_bounds__(NT) void csr_bwd_val_kernel(
     const float *__restrict__ x, int64_t ldx, const int64_t *__restrict__ crow,
     const float *__restrict__ grad, const int32_t *__restrict__ argmax,
-    const int32_t *__restrict__ argmin, const int32_t *__restrict__ pos_sel, int64_t nm,
-    float *__restrict__ val_grad, int N, int M, int vec_in)
+    const int32_t *__restrict__ argmin, const int32_t *__restrict__ pos_sel,
+    const float *__restrict__ x_sel, int64_t nm, float *__restrict__ val_grad, int N, int M, int vec_in)
 {
     __shared__ float hist[VAL_CAP];
     const int tid = threadIdx.x;
@@ -486,8 +502,9 @@ __global__ __launch_bounds__(NT) void csr_bwd_val_kernel(
                 const int64_t q1 = (int64_t)p1[r] - c0, q2 = (int64_t)p2[r] - c0;
                 p1[r] = (p1[r] >= 0 && q1 >= 0 && q1 < len) ? (int)q1 : -1;
                 p2[r] = (p2[r] >= 0 && q2 >= 0 && q2 < len) ? (int)q2 : -1;
-                x1[r] = p1[r] >= 0 ? xr[a1[r]] : 0.0f;
-                x2[r] = p2[r] >= 0 ? xr[a2[r]] : 0.0f;
+                // (the forward can hand the selected inputs over; else gather them)
+                x1[r] = p1[r] >= 0 ? (x_sel ? x_sel[o + r] : xr[a1[r]]) : 0.0f;
+                x2[r] = p2[r] >= 0 ? (x_sel ? x_sel[nm + o + r] : xr[a2[r]]) : 0.0f;
             }
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
@@ -499,6 +516,151 @@ __global__ __launch_bounds__(NT) void csr_bwd_val_kernel(
         for (int i = tid; i < len; i += NT) val_grad[c0 + i] = hist[i];
         __syncthreads();
     }
+}
+
+// The same for 16-byte aligned inputs with M a multiple of 4 (what the operators produce): 1024 threads,
+// a thread's item is one batch row x 4 consecutive CSR rows -- five 16-byte loads (the selected inputs as
+// handed over by the forward; without them up to eight single-word gathers from x, which then take two
+// thirds of the kernel's time)
+// -- so that the four threads of a batch row cover whole 64-byte sectors and sixteen waves hide each
+// other's latencies.  The entries' cells are 64-bit fixed point (mam_fixed.h): 256 batch rows pick among
+// the few entries of a pruned row, so most lanes of an LDS atomic meet a contender, which costs an fp32
+// atomic ~190 cycles per instruction and the integer one ~8 plus 2 per lane that shares an address; the sums
+// are exact and val_grad does not depend on the order of arrival.  Terms outside the window go through a
+// queue to fp32 atomics on the stored values, a window that fits almost nothing to the fp32 LDS atomics.
+constexpr int NT_V = 1024;
+constexpr int VAL_CELLS = 7168;    // entries per pass (56 KiB of 8-byte cells: with the queue under 64 KiB)
+
+__global__ __launch_bounds__(NT_V) void csr_bwd_val_vec_kernel(
+    const float *__restrict__ x, int64_t ldx, const int64_t *__restrict__ crow,
+    const float *__restrict__ grad, const int32_t *__restrict__ argmax,
+    const int32_t *__restrict__ argmin, const int32_t *__restrict__ pos_sel,
+    const float *__restrict__ x_sel, int64_t nm, float *__restrict__ val_grad, int N, int M, int span)
+{
+    using namespace fixedpoint;
+    __shared__ unsigned long long cells[VAL_CELLS];
+    __shared__ FixedQueue q;
+    __shared__ uint32_t s_max;
+    float *hist = reinterpret_cast<float *>(cells);
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.x * RB;
+    const int rows = (M - m0) < RB ? (M - m0) : RB;
+    const int64_t e_beg = crow[m0], e_end = crow[m0 + rows];
+    constexpr int QPR = RB / 4;                      // items per batch row
+    const int items = N * QPR;
+
+    // one item: batch row n, CSR rows m0 + r0 .. r0 + 3; positions relative to the pass, -1 = nothing to add
+    float4 g, s1, s2;
+    int4 u1, u2, k1, k2;
+    float x1[4], x2[4];
+    int p1[4], p2[4];
+#define MAM_VAL_LOAD(it, c0, len)                                                                    \
+    do {                                                                                             \
+        const int n_ = (it) / QPR, r0_ = ((it) % QPR) * 4;                                           \
+        const bool ok_ = (it) < items && r0_ < rows;                                                 \
+        u1 = u2 = make_int4(-1, -1, -1, -1);                                                         \
+        k1 = k2 = make_int4(0, 0, 0, 0);                                                             \
+        g = s1 = s2 = make_float4(0.f, 0.f, 0.f, 0.f);                                               \
+        if (ok_) {                                                                                   \
+            const int64_t o_ = (int64_t)n_ * M + m0 + r0_;                                           \
+            g = *reinterpret_cast<const float4 *>(grad + o_);                                        \
+            u1 = *reinterpret_cast<const int4 *>(pos_sel + o_);                                      \
+            u2 = *reinterpret_cast<const int4 *>(pos_sel + nm + o_);                                 \
+            if (x_sel) {                                                                             \
+                s1 = *reinterpret_cast<const float4 *>(x_sel + o_);                                  \
+                s2 = *reinterpret_cast<const float4 *>(x_sel + nm + o_);                             \
+            } else {                                                                                 \
+                k1 = *reinterpret_cast<const int4 *>(argmax + o_);                                   \
+                k2 = *reinterpret_cast<const int4 *>(argmin + o_);                                   \
+            }                                                                                        \
+        }                                                                                            \
+        const float sa_[4] = {s1.x, s1.y, s1.z, s1.w}, sb_[4] = {s2.x, s2.y, s2.z, s2.w};            \
+        const int pa_[4] = {u1.x, u1.y, u1.z, u1.w}, pb_[4] = {u2.x, u2.y, u2.z, u2.w};              \
+        const int ka_[4] = {k1.x, k1.y, k1.z, k1.w}, kb_[4] = {k2.x, k2.y, k2.z, k2.w};              \
+        const float *xr_ = x + (int64_t)n_ * ldx;                                                    \
+        _Pragma("unroll") for (int u_ = 0; u_ < 4; ++u_) {                                           \
+            const int64_t qa_ = (int64_t)pa_[u_] - (c0), qb_ = (int64_t)pb_[u_] - (c0);              \
+            p1[u_] = (pa_[u_] >= 0 && qa_ >= 0 && qa_ < (len)) ? (int)qa_ : -1;                      \
+            p2[u_] = (pb_[u_] >= 0 && qb_ >= 0 && qb_ < (len)) ? (int)qb_ : -1;                      \
+            x1[u_] = p1[u_] >= 0 ? (x_sel ? sa_[u_] : xr_[ka_[u_]]) : 0.0f;                          \
+            x2[u_] = p2[u_] >= 0 ? (x_sel ? sb_[u_] : xr_[kb_[u_]]) : 0.0f;                          \
+        }                                                                                            \
+    } while (0)
+
+    if (tid == 0) {
+        s_max = 0u;
+        q.count = 0;
+    }
+    __syncthreads();
+    bool fixed = span >= 8;
+    bool loaded = false;
+    int e_lo = 1;
+    {
+        const int len0 = (int)((e_end - e_beg) < VAL_CELLS ? (e_end - e_beg) : VAL_CELLS);
+        if (fixed) {
+            MAM_VAL_LOAD(tid, e_beg, len0);
+            loaded = true;
+            const float gv[4] = {g.x, g.y, g.z, g.w};
+            uint32_t mx = 0u;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t b1 = magnitude_bits(x1[u] * gv[u]), b2 = magnitude_bits(x2[u] * gv[u]);
+                mx = mx > b1 ? mx : b1;
+                mx = mx > b2 ? mx : b2;
+            }
+            const bool everything = items <= NT_V && e_end - e_beg <= VAL_CELLS;
+            fixed = make_window(workgroup_max(mx, &s_max), everything ? 0 : 4, span, e_lo);
+        }
+    }
+    for (int64_t c0 = e_beg; c0 < e_end; c0 += VAL_CELLS) {
+        const int len = (int)((e_end - c0) < VAL_CELLS ? (e_end - c0) : VAL_CELLS);
+        for (int attempt = fixed ? 0 : 1; attempt < 2; ++attempt) {
+            const bool fx = attempt == 0;
+            if (fx) for (int i = tid; i < len; i += NT_V) cells[i] = 0ull;
+            else for (int i = tid; i < len; i += NT_V) hist[i] = 0.0f;
+            __syncthreads();
+            for (int it = tid; it < items; it += NT_V) {
+                if (!loaded) MAM_VAL_LOAD(it, c0, len);
+                loaded = false;
+                const float gv[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (p1[u] >= 0) {
+                        const float t = x1[u] * gv[u];
+                        if (!fx) lds_add_sparse(&hist[p1[u]], t);
+                        else if (fixed_add(&cells[p1[u]], t, e_lo, span)) queue_push(q, p1[u], t);
+                    }
+                    if (p2[u] >= 0) {
+                        const float t = x2[u] * gv[u];
+                        if (!fx) lds_add_sparse(&hist[p2[u]], t);
+                        else if (fixed_add(&cells[p2[u]], t, e_lo, span)) queue_push(q, p2[u], t);
+                    }
+                }
+            }
+            __syncthreads();
+            const int queued = fx ? q.count : 0;
+            __syncthreads();
+            if (queued > QCAP) {
+                if (tid == 0) q.count = 0;
+                fixed = false;
+                continue;
+            }
+            float *dst = val_grad + c0;
+            if (fx) for (int i = tid; i < len; i += NT_V) dst[i] = cell_value(cells[i], e_lo);
+            else for (int i = tid; i < len; i += NT_V) dst[i] = hist[i];
+            if (queued > 0) {
+                __threadfence();
+                __syncthreads();
+                for (int i = tid; i < queued; i += NT_V)
+                    __hip_atomic_fetch_add(&dst[q.cell[i]], q.val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __syncthreads();
+                if (tid == 0) q.count = 0;
+            }
+            __syncthreads();
+            break;
+        }
+    }
+#undef MAM_VAL_LOAD
 }
 
 // Checks the CSR invariants the sparse kernels rely on; ORs the violations found into *status.
@@ -537,9 +699,9 @@ static int setup_device(int dev)
     const void *small[] = {(const void *)csr_fwd_kernel<1, false>, (const void *)csr_fwd_kernel<1, true>};
     const void *large[] = {(const void *)csr_fwd_kernel<4, false>, (const void *)csr_fwd_kernel<4, true>};
     for (const void *k : small)
-        ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 7 * ROWS * 64 * 4) == hipSuccess && ok;
+        ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 9 * ROWS * 64 * 4) == hipSuccess && ok;
     for (const void *k : large)
-        ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 7 * ROWS * 256 * 4) == hipSuccess && ok;
+        ok = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 9 * ROWS * 256 * 4) == hipSuccess && ok;
     if (!ok) {
         (void)hipGetLastError();
         return fail(MAM_ERR_LAUNCH, "could not raise the LDS limit of the CSR forward kernels");
@@ -586,8 +748,8 @@ extern "C" size_t mam_csr_fc_forward_workspace(int64_t N, int64_t K, int64_t M)
 
 extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                                   const float *val, const float *bias, float *c, int32_t *argmax,
-                                  int32_t *argmin, float *w_sel, int32_t *pos_sel, int64_t N, int64_t K,
-                                  int64_t M, int64_t nnz, void *workspace, size_t workspace_bytes,
+                                  int32_t *argmin, float *w_sel, int32_t *pos_sel, float *x_sel, int64_t N,
+                                  int64_t K, int64_t M, int64_t nnz, void *workspace, size_t workspace_bytes,
                                   void *stream)
 {
     using namespace mam;
@@ -616,17 +778,17 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
     if (rc != MAM_OK) return rc;
     const int vec_out = (M % 4 == 0) && ((uintptr_t)c % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
                         ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)w_sel % 16 == 0) &&
-                        ((uintptr_t)pos_sel % 16 == 0);
+                        ((uintptr_t)pos_sel % 16 == 0) && ((uintptr_t)x_sel % 16 == 0);
     // the lane-held entry data needs every xT row's byte offset in 32 bits
     const bool lm = (int64_t)K * ldt * 4 < ((int64_t)1 << 32);
     const dim3 grid1((unsigned)ceil_div(M, csr::ROWS), 1u);
     const int64_t gy = ceil_div(N, 256);
     if (gy > 65535) return fail(MAM_ERR_UNSUPPORTED, "N too large for the CSR forward grid");
     const dim3 grid4((unsigned)ceil_div(M, csr::ROWS), (unsigned)gy);
-    const size_t lds1 = (size_t)7 * csr::ROWS * 64 * sizeof(float), lds4 = (size_t)7 * csr::ROWS * 256 * sizeof(float);
+    const size_t lds1 = (size_t)9 * csr::ROWS * 64 * sizeof(float), lds4 = (size_t)9 * csr::ROWS * 256 * sizeof(float);
 #define MAM_CSR_LAUNCH(TI, LM, GRID, LDS)                                                                           \
     hipLaunchKernelGGL((csr::csr_fwd_kernel<TI, LM>), GRID, dim3(csr::NT_F), LDS, st, xT, (int)ldt, crow, col, val, \
-                       bias, c, argmax, argmin, w_sel, pos_sel, (int)N, (int)K, (int)M, vec_out)
+                       bias, c, argmax, argmin, w_sel, pos_sel, x_sel, (int)N, (int)K, (int)M, vec_out)
     if (N <= 64 && lm) MAM_CSR_LAUNCH(1, true, grid1, lds1);
     else if (N <= 64) MAM_CSR_LAUNCH(1, false, grid1, lds1);
     else if (lm) MAM_CSR_LAUNCH(4, true, grid4, lds4);
@@ -638,8 +800,8 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
 extern "C" int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *crow, const int64_t *col,
                                    const float *val, const float *grad, const int32_t *argmax,
                                    const int32_t *argmin, const float *w_sel, const int32_t *pos_sel,
-                                   float *x_grad, float *val_grad, int64_t N, int64_t K, int64_t M,
-                                   int64_t nnz, void *stream)
+                                   const float *x_sel, float *x_grad, float *val_grad, int64_t N, int64_t K,
+                                   int64_t M, int64_t nnz, void *stream)
 {
     using namespace mam;
     if (N < 0 || K < 0 || M < 0 || nnz < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
@@ -665,10 +827,15 @@ extern "C" int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *c
         if (val_grad) {
             const int vec_in = (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) && ((uintptr_t)argmax % 16 == 0) &&
                                ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)pos_sel % 16 == 0) &&
-                               ((N * M) % 4 == 0);
-            hipLaunchKernelGGL(csr::csr_bwd_val_kernel, dim3((unsigned)ceil_div(M, csr::RB)), dim3(csr::NT), 0, st,
-                               x, ldx, crow, grad, argmax, argmin, pos_sel, N * M, val_grad, (int)N, (int)M,
-                               vec_in);
+                               ((uintptr_t)x_sel % 16 == 0) && ((N * M) % 4 == 0);
+            if (vec_in)
+                hipLaunchKernelGGL(csr::csr_bwd_val_vec_kernel, dim3((unsigned)ceil_div(M, csr::RB)), dim3(csr::NT_V),
+                                   0, st, x, ldx, crow, grad, argmax, argmin, pos_sel, x_sel, N * M, val_grad, (int)N,
+                                   (int)M, fixedpoint::window_span(2 * N));
+            else
+                hipLaunchKernelGGL(csr::csr_bwd_val_kernel, dim3((unsigned)ceil_div(M, csr::RB)), dim3(csr::NT), 0,
+                                   st, x, ldx, crow, grad, argmax, argmin, pos_sel, x_sel, N * M, val_grad, (int)N,
+                                   (int)M, 0);
             rc = check_launch("csr_bwd_val_kernel");
         }
         const int rc_join = fork.join();

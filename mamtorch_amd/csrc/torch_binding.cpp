@@ -383,7 +383,8 @@ std::vector<at::Tensor> sparse_forward_impl(const at::Tensor &a, const at::Tenso
     auto argmin = at::empty({N, M}, a.options().dtype(at::kInt));
     at::Tensor w_sel, pos_sel;
     if (hand_over) {
-        w_sel = at::empty({2, N, M}, a.options());
+        // planes 0, 1: the selected stored values; planes 2, 3: the selected inputs
+        w_sel = at::empty({4, N, M}, a.options());
         pos_sel = at::empty({2, N, M}, a.options().dtype(at::kInt));
     }
     if (N > 0 && M > 0) {
@@ -393,8 +394,9 @@ std::vector<at::Tensor> sparse_forward_impl(const at::Tensor &a, const at::Tenso
                                     p.col.data_ptr<int64_t>(), p.val.data_ptr<float>(), nullptr,
                                     c.data_ptr<float>(), argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
                                     hand_over ? w_sel.data_ptr<float>() : nullptr,
-                                    hand_over ? pos_sel.data_ptr<int32_t>() : nullptr, N, K, M, p.val.numel(),
-                                    ws.data_ptr(), need, current_stream(a)),
+                                    hand_over ? pos_sel.data_ptr<int32_t>() : nullptr,
+                                    hand_over ? w_sel.data_ptr<float>() + 2 * N * M : nullptr, N, K, M,
+                                    p.val.numel(), ws.data_ptr(), need, current_stream(a)),
                  "mam_csr_fc_forward");
     }
     if (hand_over) return {c, argmax, argmin, w_sel, pos_sel};
@@ -427,9 +429,9 @@ std::vector<at::Tensor> sparse_fullyconnected_sel_backward(const at::Tensor &a, 
     const bool handed = w_sel.has_value() && w_sel->defined() && pos_sel.has_value() && pos_sel->defined();
     if (handed) {
         TORCH_CHECK(w_sel->scalar_type() == at::kFloat && w_sel->is_contiguous() && w_sel->dim() == 3 &&
-                        w_sel->size(0) == 2 && w_sel->size(1) == N && w_sel->size(2) == M &&
+                        (w_sel->size(0) == 2 || w_sel->size(0) == 4) && w_sel->size(1) == N && w_sel->size(2) == M &&
                         w_sel->device() == a.device(),
-                    "w_sel must be a contiguous float32 (2, batch, out_features) tensor on a's device");
+                    "w_sel must be a contiguous float32 (2 or 4, batch, out_features) tensor on a's device");
         TORCH_CHECK(pos_sel->scalar_type() == at::kInt && pos_sel->is_contiguous() && pos_sel->dim() == 3 &&
                         pos_sel->size(0) == 2 && pos_sel->size(1) == N && pos_sel->size(2) == M &&
                         pos_sel->device() == a.device(),
@@ -443,8 +445,10 @@ std::vector<at::Tensor> sparse_fullyconnected_sel_backward(const at::Tensor &a, 
                                  p.col.data_ptr<int64_t>(), p.val.data_ptr<float>(), g.data_ptr<float>(),
                                  argmax.data_ptr<int32_t>(), argmin.data_ptr<int32_t>(),
                                  handed ? w_sel->data_ptr<float>() : nullptr,
-                                 handed ? pos_sel->data_ptr<int32_t>() : nullptr, a_grad.data_ptr<float>(),
-                                 val_grad.data_ptr<float>(), N, K, M, p.val.numel(), current_stream(a)),
+                                 handed ? pos_sel->data_ptr<int32_t>() : nullptr,
+                                 handed && w_sel->size(0) == 4 ? w_sel->data_ptr<float>() + 2 * N * M : nullptr,
+                                 a_grad.data_ptr<float>(), val_grad.data_ptr<float>(), N, K, M, p.val.numel(),
+                                 current_stream(a)),
              "mam_csr_fc_backward");
     return {a_grad, val_grad};
 }

@@ -95,10 +95,11 @@ def test_sparse_step_replays():
     gs = torch.empty(N, M, device=dev)
     w_sel = torch.empty(2, N, M, device=dev)
     pos_sel = torch.empty(2, N, M, dtype=torch.int32, device=dev)
+    x_sel = torch.empty(2, N, M, device=dev)
 
     def step():
-        c, amax, amin = capi.csr_fc_forward(xs, *parts, M, None, w_sel, pos_sel)
-        xg, vg = capi.csr_fc_backward(xs, *parts, gs, amax, amin, w_sel, pos_sel)
+        c, amax, amin = capi.csr_fc_forward(xs, *parts, M, None, w_sel, pos_sel, x_sel)
+        xg, vg = capi.csr_fc_backward(xs, *parts, gs, amax, amin, w_sel, pos_sel, x_sel)
         return c, amax, amin, xg, vg
 
     cases = [random_case(N, K, M, seed=20 + s) for s in range(3)]

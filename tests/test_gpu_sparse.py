@@ -22,7 +22,8 @@ def _forward_backward(x, dense, crow, col, val, what, bias=None):
     parts = [t.to(dev) for t in (crow, col, val)]
     w_sel = torch.full((2, N, M), 7.0, dtype=torch.float32, device=dev)
     pos_sel = torch.full((2, N, M), -7, dtype=torch.int32, device=dev)
-    c, amax, amin = capi.csr_fc_forward(xd, *parts, M, None if bias is None else bias.to(dev), w_sel, pos_sel)
+    x_sel = torch.full((2, N, M), 7.0, dtype=torch.float32, device=dev)
+    c, amax, amin = capi.csr_fc_forward(xd, *parts, M, None if bias is None else bias.to(dev), w_sel, pos_sel, x_sel)
     c2, amax2, amin2 = capi.csr_fc_forward(xd, *parts, M, None if bias is None else bias.to(dev))
     torch.cuda.synchronize()
     assert_bits_equal(c.cpu().numpy(), want[0], what + " c")
@@ -43,17 +44,23 @@ def _forward_backward(x, dense, crow, col, val, what, bias=None):
     ws = w_sel.cpu().numpy()
     assert_bits_equal(ws[stored], val.numpy()[pos[stored]], what + " w_sel")
     assert (ws[~stored] == 0).all()
+    # ... and the selected inputs x[n, selected column] (0 where an implicit zero was selected)
+    xs = x_sel.cpu().numpy()
+    n_of = np.broadcast_to(np.arange(N)[None, :, None], (2, N, M))
+    assert_bits_equal(xs[stored], x.numpy()[n_of[stored], sel[stored]], what + " x_sel")
+    assert (xs[~stored] == 0).all()
     grad = torch.randn(N, M, generator=torch.Generator().manual_seed(1))
     xo, vo = oracle.csr_backward(x.numpy(), crow.numpy(), col.numpy(), val.numpy(), grad.numpy(), want[1], want[2])
     # rtol 1e-5 plus the rounding floor of an fp32 sum in any order: 2^-22 x the sum of |terms| of the
     # cell, measured by the oracle's backward over absolute values
     xa, va = oracle.csr_backward(np.abs(x.numpy()), crow.numpy(), col.numpy(), np.abs(val.numpy()),
                                  np.abs(grad.numpy()), want[1], want[2])
-    for handed in (False, True):
+    for handed in (0, 1, 2):
         xg, vg = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin,
-                                      w_sel if handed else None, pos_sel if handed else None)
+                                      w_sel if handed else None, pos_sel if handed else None,
+                                      x_sel if handed == 2 else None)
         torch.cuda.synchronize()
-        tag = what + (" (hand-over)" if handed else " (search)")
+        tag = what + (" (search)", " (hand-over)", " (hand-over with inputs)")[handed]
         for got, wanted, floor, name in ((xg, xo, xa, "x_grad"), (vg, vo, va, "val_grad")):
             err = np.abs(got.cpu().numpy().astype(np.float64) - wanted)
             bound = 1e-5 * np.abs(wanted) + 2.0 ** -22 * floor + 1e-30
@@ -185,10 +192,12 @@ def test_config5_full_size_equals_dense_kernel(density):
     grad = torch.randn(N, M, generator=torch.Generator().manual_seed(6))
     w_sel = torch.empty((2, N, M), dtype=torch.float32, device=dev)
     pos_sel = torch.empty((2, N, M), dtype=torch.int32, device=dev)
-    c3, amax3, amin3 = capi.csr_fc_forward(xd, *parts, M, None, w_sel, pos_sel)
+    x_sel = torch.empty((2, N, M), dtype=torch.float32, device=dev)
+    c3, amax3, amin3 = capi.csr_fc_forward(xd, *parts, M, None, w_sel, pos_sel, x_sel)
     assert torch.equal(c3.view(torch.int32), cd.view(torch.int32)) and torch.equal(amax3, dmax)
     xg, vg = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin)
     xg2, vg2 = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin, w_sel, pos_sel)
+    xg3, vg3 = capi.csr_fc_backward(xd, *parts, grad.to(dev), amax, amin, w_sel, pos_sel, x_sel)
     xdg, wdg = capi.fc_backward(xd, dense.to(dev), grad.to(dev), amax, amin, capi.W_MK)
     torch.cuda.synchronize()
     # two fp32 summation orders of the same terms: each may be off by the rounding floor of the
@@ -197,7 +206,7 @@ def test_config5_full_size_equals_dense_kernel(density):
     torch.cuda.synchronize()
     rws = torch.repeat_interleave(torch.arange(M), crow[1:] - crow[:-1]).to(dev)
     want_v, abs_v = wdg[rws, col.to(dev)], wabs[rws, col.to(dev)]
-    for got_x, got_v in ((xg, vg), (xg2, vg2)):
+    for got_x, got_v in ((xg, vg), (xg2, vg2), (xg3, vg3)):
         assert bool(((got_x - xdg).abs() <= 1e-5 * xdg.abs() + 2.0 ** -21 * xabs).all())
         assert bool(((got_v - want_v).abs() <= 1e-5 * want_v.abs() + 2.0 ** -21 * abs_v).all())
 
