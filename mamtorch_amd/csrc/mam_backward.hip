@@ -563,13 +563,15 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
     const int cus = num_cus();
     // 64-bit fixed-point cells: room for 2 * M * planes terms of 24 + span - 1 bits each, and one bit to spare
     const int span = window_span(2 * M * planes);
-    const bool x_rows = N >= 2048 && K * 16 <= 64 * 1024 && (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
+    const bool x_rows = N >= 2048 && K * 16 <= ((int64_t)lds_cap * 4 - 8192 < 64 * 1024 ? (int64_t)lds_cap * 4 - 8192 : 64 * 1024) && (M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
                         ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) &&
                         ((uintptr_t)w_sel % 16 == 0);
     if (x_grad && x_rows) {
         // as many rows per workgroup (2 to 16) as fit 64 KiB of LDS in 8-byte cells
+        // (the queue and the window's scratch are static LDS on top of the cells: 8 KiB kept free for them)
+        const int64_t rows_budget = kRowsLdsBytes < (int64_t)lds_cap * 4 - 8192 ? kRowsLdsBytes : (int64_t)lds_cap * 4 - 8192;
         int log2r = 1;
-        while (log2r < 4 && ((int64_t)2 << log2r) * K * 8 <= kRowsLdsBytes) ++log2r;
+        while (log2r < 4 && ((int64_t)2 << log2r) * K * 8 <= rows_budget) ++log2r;
         const int R = 1 << log2r;
         hipLaunchKernelGGL((mam_bwd_x_rows_kernel<LAYOUT>), dim3((unsigned)ceil_div(N, R)), dim3(NT_W),
                            (size_t)R * K * 8, st, w, ldw, grad, argmax, argmin, w_sel, N * M, x_grad,
@@ -577,7 +579,8 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         rc = check_launch("mam_bwd_x_rows_kernel");
         if (rc != MAM_OK) return rc;
     } else if (x_grad) {
-        const int kc = (int)(K < lds_cap / 2 ? K : lds_cap / 2);
+        const int cells_cap = (lds_cap - 2048) / 2;     // 8-byte cells, 8 KiB kept free for the static LDS
+        const int kc = (int)(K < cells_cap ? K : cells_cap);
         hipLaunchKernelGGL((mam_bwd_x_kernel<LAYOUT>), dim3((unsigned)N), dim3(NT_X),
                            (size_t)kc * 8, st, w, ldw, grad, argmax, argmin, w_sel, N * M,
                            x_grad, (int)K, (int)M, kc, planes, span);
@@ -649,7 +652,8 @@ int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t
 {
     const int dev = ensure_device();
     if (dev < 0) return dev;
-    const int kc = (int)(K < g_lds_floats[dev] / 2 ? K : g_lds_floats[dev] / 2);
+    const int cells_cap = (g_lds_floats[dev] - 2048) / 2;
+    const int kc = (int)(K < cells_cap ? K : cells_cap);
     hipLaunchKernelGGL((mam_bwd_x_kernel<MAM_W_MK>), dim3((unsigned)N), dim3(NT_X), (size_t)kc * 8,
                        st, (const float *)nullptr, (int64_t)0, grad, argmax, argmin, w_sel, N * M, x_grad, (int)K,
                        (int)M, kc, 1, window_span(2 * M));
