@@ -67,7 +67,7 @@ def test_known_answer_selection_count():
     lit = torch_port.selection_count_reference(torch.tensor(amax), torch.tensor(amin),
                                                torch.zeros((kat["M"], kat["K"]), dtype=torch.int32))
     np.testing.assert_array_equal(lit.numpy(), _arr(kat["ref_max_count"], np.int32))
-    # the survey's example: three hits on one cell add 1
+    # three hits on one cell add 1, not 3
     z = torch.zeros(3, 4, dtype=torch.int32)
     z[torch.tensor([0, 0, 0, 1]), torch.tensor([2, 2, 2, 3])] += 1
     assert z.tolist() == [[0, 0, 1, 0], [0, 0, 0, 1], [0, 0, 0, 0]]
