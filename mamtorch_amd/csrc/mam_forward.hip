@@ -1359,8 +1359,8 @@ extern "C" int mam_fc_forward_describe(const float *x, int64_t ldx, const float 
     const fwd::Params &p = plan.p;
     const char *what = with_indices ? "args" : "values";
     if (plan.use_sx)
-        snprintf(text, text_bytes, "mam_fwd_sx_kernel<%s%s> %d x %d tiles of 32 x 128", what, p.splits > 1 ? ", split" : "",
-                 p.tiles_n, p.tiles_m);
+        snprintf(text, text_bytes, "mam_fwd_sx_kernel<%s%s%s> %d x %d tiles of 32 x 128", what, p.splits > 1 ? ", split" : "",
+                 K % fwd::sx::KT != 0 ? ", partial last k tile" : "", p.tiles_n, p.tiles_m);
     else
         snprintf(text, text_bytes, "mam_fwd_kernel<%s, %s> %d x %d tiles of 64 x 128", w_layout == MAM_W_MK ? "(M,K)" : "(K,M)",
                  what, p.tiles_n, p.tiles_m);
