@@ -57,9 +57,16 @@ __device__ __forceinline__ void queue_push(FixedQueue &q, int cell, float t)
     }
 }
 
+// The cell as fp32: through fp64, whose conversions and scaling are single instructions (an int64 -> fp32
+// conversion is a ~20-instruction sequence, and a slab has one cell per output element).  The fp64 value is
+// exact below 2^53 in magnitude and rounded once to fp32; a larger sum (dozens of terms of the window's top
+// binades in one cell) is first rounded to 53 bits, which can move the fp32 result by one unit in the last
+// place only when that rounding lands exactly on an fp32 tie.
 __device__ __forceinline__ float cell_value(unsigned long long c, int e_lo)
 {
-    return ldexpf((float)(long long)c, e_lo - 150);
+    const double hi = (double)(int)(c >> 32) * 4294967296.0;
+    const double lo = (double)(unsigned int)c;
+    return (float)ldexp(hi + lo, e_lo - 150);
 }
 
 __device__ __forceinline__ uint32_t magnitude_bits(float t) { return __float_as_uint(t) & 0x7fffffffu; }
