@@ -227,12 +227,23 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
         q.count = 0;
     }
     __syncthreads();
-    bool fixed = span >= 8 && w_sel != nullptr;    // (a window needs the terms of the first trip: handed-over weights)
+    bool fixed = span >= 8;
     int e_lo = 1;
     if (fixed) {
         MAM_LOAD_ITEM(0, m_first);
         uint32_t mx = 0u;
         if (row_ok && m_first < M) {
+            if (!w_sel) {     // no hand-over: the first trip's weights are gathered for the window as well
+                const int k1[4] = {i1.x, i1.y, i1.z, i1.w}, k2[4] = {i2.x, i2.y, i2.z, i2.w};
+                float w1[4], w2[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    w1[u] = (unsigned)k1[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k1[u], m_first + u) : 0.0f;
+                    w2[u] = (unsigned)k2[u] < (unsigned)K ? load_w<LAYOUT>(w, ldw, k2[u], m_first + u) : 0.0f;
+                }
+                s1 = make_float4(w1[0], w1[1], w1[2], w1[3]);
+                s2 = make_float4(w2[0], w2[1], w2[2], w2[3]);
+            }
             const float t[8] = {s1.x * g.x, s1.y * g.y, s1.z * g.z, s1.w * g.w, s2.x * g.x, s2.y * g.y, s2.z * g.z, s2.w * g.w};
 #pragma unroll
             for (int u = 0; u < 8; ++u) {

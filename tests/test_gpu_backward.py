@@ -314,3 +314,8 @@ def test_x_grad_is_reproducible_bit_for_bit(shape):
     # and it is the correctly rounded exact sum: fp64 accumulation of the fp32 terms, rounded once
     xo, _ = oracle.backward(x.numpy(), w.numpy(), grad.numpy(), amax.cpu().numpy(), amin.cpu().numpy(), oracle.W_MK)
     np.testing.assert_array_equal(first.cpu().numpy(), xo.astype(np.float32))
+    # the same without the hand-over (weights gathered by index), in both weight layouts
+    gathered, _ = capi.fc_backward(xd, wd, gd, amax, amin, capi.W_MK, want_w=False)
+    assert torch.equal(first, gathered)
+    gathered, _ = capi.fc_backward(xd, wd.T.contiguous(), gd, amax, amin, capi.W_KM, want_w=False)
+    assert torch.equal(first, gathered)
