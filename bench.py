@@ -17,6 +17,7 @@ restatement of the reference's CPU path (oracle/torch_port.py) timed on a bounde
 Other workloads (`--workload`), same JSON layout, used for the tables in the design notes:
   vit_mlp            12608 rows through MAM FC 768->3072 and MAM FC 3072->768, forward + backward
   inference_m{1024,4096,16384}   batch 16384, in 4096, forward with indices only
+  config1            batch 64, 784 -> 256: forward + backward + selection count (launch-latency bound)
   values_headline    headline shape, values-only forward
   sparse_d{10,03,01} 4096x4096 weight pruned to 10 % / 3 % / 1 %, batch 256, CSR forward + backward
   spmm_d{30,10,01}   sum-of-products SpMM (cusparsemm): 4096x4096 CSR with 30 % / 10 % / 1 % stored, times a
@@ -52,7 +53,7 @@ RAMP_MIN_CALLS = 300          # untimed phase calls before the counted warm-up: 
 RAMP_MIN_SECONDS = 0.3
 RAMP_MAX_SECONDS = 3.0
 
-WORKLOADS = ("headline", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
+WORKLOADS = ("headline", "config1", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
              "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01", "prune_csr")
 
 
@@ -244,6 +245,15 @@ def run_dense(torch, capi, lib, dev, args):
                 "backward (grad_x, grad_W) + selection-count accumulation; x~N(0,1), W~U(-1/64,1/64), "
                 "grad_out~N(0,1), seed 0; weight in (out,in) layout") if wl == "headline" else \
                "MAM FullyConnected fp32 batch 256 in 4096 out 4096: values-only forward; x~N(0,1), W~U(-1/64,1/64)"
+    elif wl == "config1":
+        N, K, M = 64, 784, 256
+        x = torch.randn(N, K, generator=gen)
+        w = (torch.rand(M, K, generator=gen) * 2 - 1) / 28.0       # Kaiming-uniform(a=sqrt 5), fan_in 784
+        g = torch.randn(N, M, generator=gen)
+        shapes = [(x, w, g)]
+        backward, count, values = True, True, False
+        text = ("MAM FullyConnected fp32 batch 64 in 784 out 256 (the small configuration the CPU can run whole): "
+                "forward with argmax/argmin + backward + selection count; launch-latency bound")
     elif wl == "vit_mlp":
         N = 12608
         shapes = []
@@ -507,7 +517,7 @@ def main():
         print("bench.py measures one GPU: the MAM hot path has no multi-GPU part in this build "
               "(--gpus %d refused)" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    small = args.workload in ("headline", "values_headline", "prune_csr") or args.workload.startswith("sparse")
+    small = args.workload in ("headline", "config1", "values_headline", "prune_csr") or args.workload.startswith("sparse")
     if args.workload.startswith("spmm"):
         args.steps = 50 if args.steps is None else args.steps
         args.warmup = 20 if args.warmup is None else args.warmup
