@@ -158,15 +158,15 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
                 continue;
             }
             float *dst = x_grad + (int64_t)n * K;
-            if (fx) for (int i = tid; i < kn; i += NT_X) dst[k0 + i] = cell_value(cells[i], e_lo);
-            else for (int i = tid; i < kn; i += NT_X) dst[k0 + i] = hist[i];
             if (queued > 0) {
-                __threadfence();
-                __syncthreads();
-                for (int i = tid; i < queued; i += NT_X)
-                    __hip_atomic_fetch_add(&dst[q.cell[i]], q.val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __syncthreads();
+                settle_queue<NT_X>(cells, kn, q, queued, e_lo, k0);
+                const double *d = reinterpret_cast<const double *>(cells);
+                for (int i = tid; i < kn; i += NT_X) dst[k0 + i] = (float)d[i];
                 if (tid == 0) q.count = 0;
+            } else if (fx) {
+                for (int i = tid; i < kn; i += NT_X) dst[k0 + i] = cell_value(cells[i], e_lo);
+            } else {
+                for (int i = tid; i < kn; i += NT_X) dst[k0 + i] = hist[i];
             }
             __syncthreads();
             break;
@@ -298,14 +298,14 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
         const int queued = fx ? q.count : 0;
         __syncthreads();
         if (queued > QCAP) continue;      // the window was a bad guess: once more with fp32 atomics
-        if (fx) for (int i = tid; i < rows * K; i += NT_W) dst[i] = cell_value(cells[i], e_lo);
-        else for (int i = tid; i < rows * K; i += NT_W) dst[i] = hist[i];
         if (queued > 0) {
-            __threadfence();
-            __syncthreads();
-            for (int i = tid; i < queued; i += NT_W)
-                if (q.cell[i] < rows * K)
-                    __hip_atomic_fetch_add(&dst[q.cell[i]], q.val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            settle_queue<NT_W>(cells, R * K, q, queued, e_lo, 0);
+            const double *d = reinterpret_cast<const double *>(cells);
+            for (int i = tid; i < rows * K; i += NT_W) dst[i] = (float)d[i];
+        } else if (fx) {
+            for (int i = tid; i < rows * K; i += NT_W) dst[i] = cell_value(cells[i], e_lo);
+        } else {
+            for (int i = tid; i < rows * K; i += NT_W) dst[i] = hist[i];
         }
         break;
     }

@@ -527,7 +527,7 @@ __global__ __launch_bounds__(NT) void csr_bwd_val_kernel(
 // the few entries of a pruned row, so most lanes of an LDS atomic meet a contender, which costs an fp32
 // atomic ~190 cycles per instruction and the integer one ~8 plus 2 per lane that shares an address; the sums
 // are exact and val_grad does not depend on the order of arrival.  Terms outside the window go through a
-// queue to fp32 atomics on the stored values, a window that fits almost nothing to the fp32 LDS atomics.
+// queue and are added in fp64 before the one rounding, a window that fits almost nothing to the fp32 LDS atomics.
 constexpr int NT_V = 1024;
 constexpr int VAL_CELLS = 7168;    // entries per pass (56 KiB of 8-byte cells: with the queue under 64 KiB)
 
@@ -646,15 +646,15 @@ __global__ __launch_bounds__(NT_V) void csr_bwd_val_vec_kernel(
                 continue;
             }
             float *dst = val_grad + c0;
-            if (fx) for (int i = tid; i < len; i += NT_V) dst[i] = cell_value(cells[i], e_lo);
-            else for (int i = tid; i < len; i += NT_V) dst[i] = hist[i];
             if (queued > 0) {
-                __threadfence();
-                __syncthreads();
-                for (int i = tid; i < queued; i += NT_V)
-                    __hip_atomic_fetch_add(&dst[q.cell[i]], q.val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __syncthreads();
+                settle_queue<NT_V>(cells, len, q, queued, e_lo, 0);
+                const double *d = reinterpret_cast<const double *>(cells);
+                for (int i = tid; i < len; i += NT_V) dst[i] = (float)d[i];
                 if (tid == 0) q.count = 0;
+            } else if (fx) {
+                for (int i = tid; i < len; i += NT_V) dst[i] = cell_value(cells[i], e_lo);
+            } else {
+                for (int i = tid; i < len; i += NT_V) dst[i] = hist[i];
             }
             __syncthreads();
             break;

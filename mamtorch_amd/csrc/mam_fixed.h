@@ -14,7 +14,7 @@ namespace fixedpoint {
 // ~190.  span leaves room for every term a cell can receive (2 * M * planes), so the sum cannot overflow.
 // The window is placed by the largest term of the workgroup's first trip (plus 4 binades where that is
 // not the whole row).  The rare term outside it (tiny, huge, denormal, inf, nan) is parked in a small LDS
-// queue and added to the stored slab with fp32 atomics afterwards; if the queue overflows -- a first trip
+// queue and added, in fp64, before the slab is rounded and stored; if the queue overflows -- a first trip
 // that says nothing about the rest -- the workgroup starts over with the fp32 LDS atomics.
 constexpr int QCAP = 512;
 struct FixedQueue {
@@ -57,16 +57,35 @@ __device__ __forceinline__ void queue_push(FixedQueue &q, int cell, float t)
     }
 }
 
-// The cell as fp32: through fp64, whose conversions and scaling are single instructions (an int64 -> fp32
-// conversion is a ~20-instruction sequence, and a slab has one cell per output element).  The fp64 value is
-// exact below 2^53 in magnitude and rounded once to fp32; a larger sum (dozens of terms of the window's top
-// binades in one cell) is first rounded to 53 bits, which can move the fp32 result by one unit in the last
-// place only when that rounding lands exactly on an fp32 tie.
-__device__ __forceinline__ float cell_value(unsigned long long c, int e_lo)
+// The cell as fp64 and as fp32: through fp64, whose conversions and scaling are single instructions (an
+// int64 -> fp32 conversion is a ~20-instruction sequence, and a slab has one cell per output element).  The
+// fp64 value is exact below 2^53 in magnitude and rounded once to fp32; a larger sum (dozens of terms of the
+// window's top binades in one cell) is first rounded to 53 bits, which can move the fp32 result by one unit in
+// the last place only when that rounding lands exactly on an fp32 tie.
+__device__ __forceinline__ double cell_double(unsigned long long c, int e_lo)
 {
     const double hi = (double)(int)(c >> 32) * 4294967296.0;
     const double lo = (double)(unsigned int)c;
-    return (float)ldexp(hi + lo, e_lo - 150);
+    return ldexp(hi + lo, e_lo - 150);
+}
+__device__ __forceinline__ float cell_value(unsigned long long c, int e_lo) { return (float)cell_double(c, e_lo); }
+
+// A slab with queued terms: every cell is replaced by its fp64 value, in place, and the queued terms (each
+// fp32, outside the window) are added in fp64, so that the one rounding to fp32 happens after them as well;
+// the caller then stores (float) of the doubles.  Queue entries name cells as `cell_base` + index.
+template <int NT>
+__device__ __forceinline__ void settle_queue(unsigned long long *cells, int ncells, const FixedQueue &q, int queued,
+                                             int e_lo, int cell_base)
+{
+    double *d = reinterpret_cast<double *>(cells);
+    for (int i = threadIdx.x; i < ncells; i += NT) d[i] = cell_double(cells[i], e_lo);
+    __syncthreads();
+    for (int i = threadIdx.x; i < queued; i += NT) {
+        const int idx = q.cell[i] - cell_base;
+        if ((unsigned)idx < (unsigned)ncells)
+            __hip_atomic_fetch_add(&d[idx], (double)q.val[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    __syncthreads();
 }
 
 __device__ __forceinline__ uint32_t magnitude_bits(float t) { return __float_as_uint(t) & 0x7fffffffu; }

@@ -67,7 +67,50 @@ def test_forward_and_backward_over_ranges(N, K, M, range_len):
             err = np.abs(got.astype(np.float64) - wanted)
             assert (err <= 1e-5 * np.abs(wanted) + 2.0 ** -22 * floor + 1e-30).all(), tag + " " + name
         xg_only, none = capi.fc_backward_ranges(xd, wd, gd, amax, amin, range_len, layout, want_w=False)
-        assert none is None and torch.allclose(xg_only, xg, rtol=1e-4, atol=1e-5)   # LDS atomics: order varies
+        assert none is None and torch.equal(xg_only, xg)     # exact sums: no dependence on the order of arrival
+
+
+def test_headline_shape_with_the_modules_splits():
+    """Config 2 (batch 256, 4096 -> 4096) with splits = 4: the oracle on a sample of batch rows, and on all rows
+    the property that the output is the sum over the ranges of (max + min) of the selected products."""
+    from mamtorch_amd import capi
+
+    N, K, M, range_len = 256, 4096, 4096, 1024
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(N, K, generator=g)
+    w = (torch.rand(M, K, generator=g) * 2 - 1) / 64.0
+    grad = torch.randn(N, M, generator=g)
+    xd, wd, gd = x.to(DEV), w.to(DEV), grad.to(DEV)
+    c, amax, amin = capi.fc_forward_ranges(xd, wd, range_len, capi.W_MK, None)
+    torch.cuda.synchronize()
+    rows = torch.arange(0, N, 16)
+    want_c, want_max, want_min = _oracle_ranges(x[rows].numpy(), w.numpy(), None, range_len)
+    assert_bits_equal(c[rows.to(DEV)].cpu().numpy(), want_c, "headline splits c")
+    assert_index_equal(amax[:, rows.to(DEV)].cpu().numpy(), want_max, "headline splits argmax")
+    assert_index_equal(amin[:, rows.to(DEV)].cpu().numpy(), want_min, "headline splits argmin")
+    # all rows: c = sum over ranges, in ascending order, of x[n, argmax] * w[m, argmax] + x[n, argmin] * w[m, argmin]
+    total = None
+    cols = torch.arange(M, device=DEV)[None, :]
+    nrows = torch.arange(N, device=DEV)[:, None]
+    for r in range(K // range_len):
+        i1, i2 = amax[r].long(), amin[r].long()
+        assert int(i1.min()) >= r * range_len and int(i1.max()) < (r + 1) * range_len
+        part = xd[nrows, i1] * wd[cols, i1] + xd[nrows, i2] * wd[cols, i2]
+        total = part if total is None else total + part
+    assert torch.equal(total.view(torch.int32), c.view(torch.int32))
+    # backward: each range routes grad to its own two positions; sums of the gradients match the closed form
+    xg, wg = capi.fc_backward_ranges(xd, wd, gd, amax, amin, range_len, capi.W_MK)
+    torch.cuda.synchronize()
+    want_x = torch.zeros(N, K, dtype=torch.float64, device=DEV)
+    want_w = torch.zeros(M, K, dtype=torch.float64, device=DEV)
+    for r in range(K // range_len):
+        for idx in (amax[r].long(), amin[r].long()):
+            want_x.scatter_add_(1, idx, (gd * wd[cols, idx]).double())
+            want_w.scatter_add_(1, idx.T.contiguous(), (gd * xd[nrows, idx]).double().T.contiguous())
+    bad = (xg != want_x.float())
+    assert not bool(bad.any()), "x_grad: %d cells differ from the exact sum rounded once, worst %g" % (
+        int(bad.sum()), float((xg.double() - want_x).abs().max()))
+    assert torch.allclose(wg.double(), want_w, rtol=1e-5, atol=1e-5)
 
 
 def test_zero_extremes_inside_ranges_keep_their_sign():
