@@ -827,7 +827,6 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     using C = sx::Cfg<TJ>;
     __shared__ __attribute__((aligned(16))) float tile_a[C::TILE_FLOATS];
     __shared__ __attribute__((aligned(16))) float tile_b[C::TILE_FLOATS];
-    __shared__ uint32_t doff_s[C::DMA_PER_WAVE * sx::NT];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -869,8 +868,10 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
         xr[i] = (const_f32 *)(p.x + (int64_t)row * p.ldx + kb);
     }
 
-    // per-lane byte offsets of this wave's direct-to-LDS loads, kept in LDS
-    const uint32_t *doff = doff_s + tid;
+    // per-lane byte offsets of this wave's direct-to-LDS loads.  They stay in registers, and the
+    // loads take them as the 32-bit offset of the (scalar base + vector offset) addressing form: formed
+    // per lane in 64 bits, the addresses were 16 64-bit adds per tile.
+    uint32_t doff[C::DMA_PER_WAVE];
 #pragma unroll
     for (int t = 0; t < C::DMA_PER_WAVE; ++t) {
         const int inst = wave + (sx::NT / 64) * t;
@@ -878,16 +879,19 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
         // the k chunk that belongs at this LDS position
         const int chunk = (lane % sx::CHUNKS) ^ ((r / sx::RPB) & (sx::CHUNKS - 1));
         const int rc = ((col0 + r) < p.M ? (col0 + r) : (p.M - 1)) - col0;
-        doff_s[t * sx::NT + tid] = (uint32_t)(rc * (int)p.ldw + chunk * 4) * 4u;
+        doff[t] = (uint32_t)(rc * (int)p.ldw + chunk * 4) * 4u;
     }
     const int sw = (lane / sx::RPB) & (sx::CHUNKS - 1);   // the same for neurons lane + 64 j
     const int wbase = lane * sx::KT;     // floats; neuron lane + 64 j is 64 j * KT further
 
     auto dma = [&](const char *wk, float *tile) {
+        asm volatile("" : "+s"(wk));     // one scalar base for the loads of this tile
 #pragma unroll
         for (int t = 0; t < C::DMA_PER_WAVE; ++t) {
             const int inst = wave + (sx::NT / 64) * t;
-            const char *src = wk + (uint64_t)doff[t * sx::NT];
+            uint32_t off = doff[t];
+            asm volatile("" : "+v"(off));    // keeps the zero-extension next to the load (no hoisted 64-bit copy)
+            const char *src = wk + (uint64_t)off;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                              (__attribute__((address_space(3))) void *)(tile + inst * 256), 16, 0, 0);
         }
@@ -947,7 +951,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
                 const int r = inst * (64 / sx::CHUNKS) + lane / sx::CHUNKS;
                 const int chunk = (lane % sx::CHUNKS) ^ ((r / sx::RPB) & (sx::CHUNKS - 1));
                 if (chunk * 4 < tail_groups * G) {
-                    const char *src = wk + (uint64_t)doff[u * sx::NT];
+                    const char *src = wk + (uint64_t)doff[u];
                     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                                      (__attribute__((address_space(3))) void *)(tile + inst * 256), 16, 0, 0);
                 }
