@@ -48,16 +48,21 @@ extern "C" {
                                  likewise for min (the retired convolution modules' literal rule)        */
 
 /* Run-time switches for mam_set_option().  Their initial values come from the environment variables of
- * the same names (MAM_FORWARD_TILING = auto | wide, MAM_BACKWARD_FORK = 0 | 1), read once when the
+ * the same names (MAM_FORWARD_TILING = auto | wide, MAM_BACKWARD_FORK = 0 | 1, MAM_BACKWARD_ONE_LAUNCH = 0 | 1), read once when the
  * library is loaded. */
 #define MAM_OPT_FORWARD_TILING 0 /* which dense forward tiling serves a call                      */
 #define MAM_OPT_BACKWARD_FORK 1  /* x_grad on the library's second stream beside w_grad           */
-#define MAM_OPT_COUNT_ 2
+#define MAM_OPT_BACKWARD_ONE_LAUNCH 2 /* both gradients in one launch where the shape allows it    */
+#define MAM_OPT_COUNT_ 3
 #define MAM_FORWARD_TILING_AUTO 0 /* wave-uniform-rows tiling where the layout allows it           */
 #define MAM_FORWARD_TILING_WIDE 1 /* every call on the general 64 x 128 tiling                     */
 #define MAM_BACKWARD_FORK_AUTO (-1) /* from 2^22 outputs on, and under stream capture from 2^16   */
 #define MAM_BACKWARD_FORK_OFF 0
 #define MAM_BACKWARD_FORK_ON 1
+#define MAM_BACKWARD_ONE_LAUNCH_OFF 0
+#define MAM_BACKWARD_ONE_LAUNCH_AUTO 1 /* small calls only (<= 2^16 outputs), where the launches are the cost */
+#define MAM_BACKWARD_ONE_LAUNCH_ON 2   /* wherever the shape allows it: (M,K) weights, 16-byte aligned operands,
+                                          batch below 2 x CUs, K <= 4096 */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int mam_version(void);

@@ -17,6 +17,7 @@ PRUNE_WEIGHT_TIMES = 1
 PRUNE_COUNT = 2
 OPT_FORWARD_TILING = 0
 OPT_BACKWARD_FORK = 1
+OPT_BACKWARD_ONE_LAUNCH = 2
 FORWARD_TILING_AUTO = 0
 FORWARD_TILING_WIDE = 1
 BACKWARD_FORK_AUTO = -1

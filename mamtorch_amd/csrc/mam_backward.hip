@@ -53,20 +53,19 @@ __device__ __forceinline__ void lds_add_sparse(float *addr, float v)
     if (!done) lds_add(addr, v);
 }
 
+// The work of one workgroup of mam_bwd_x_kernel: batch row n, its kc cells in `cells`.
 template <int LAYOUT>
-__global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
-    const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
+__device__ __forceinline__ void bwd_x_body(
+    unsigned long long *cells, int n, const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
     const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int K, int M, int kc, int planes,
     int span)
 {
     // planes > 1 (the module's `splits`): argmax / argmin are [plane][N*M] arrays of absolute k, one pair
     // per K range, w_sel (if any) [plane][2][N*M]; every plane scatters the same grad
-    extern __shared__ unsigned long long cells[];      // kc cells; the fp32 fallback uses the same bytes
     __shared__ FixedQueue q;
     __shared__ uint32_t s_max;
-    float *hist = reinterpret_cast<float *>(cells);
-    const int n = blockIdx.x;
+    float *hist = reinterpret_cast<float *>(cells);   // kc cells; the fp32 fallback uses the same bytes
     const int tid = threadIdx.x;
     const float *g_row = grad + (int64_t)n * M;
 
@@ -172,6 +171,17 @@ __global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
             break;
         }
     }
+}
+
+template <int LAYOUT>
+__global__ __launch_bounds__(NT_X) void mam_bwd_x_kernel(
+    const float *__restrict__ w, int64_t ldw, const float *__restrict__ grad,
+    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
+    const float *__restrict__ w_sel, int64_t nm, float *__restrict__ x_grad, int K, int M, int kc, int planes,
+    int span)
+{
+    extern __shared__ unsigned long long cells[];
+    bwd_x_body<LAYOUT>(cells, blockIdx.x, w, ldw, grad, argmax, argmin, w_sel, nm, x_grad, K, M, kc, planes, span);
 }
 
 // x_grad for large batches: a workgroup owns R = 2 .. 16 batch rows with their whole K cells in LDS,
@@ -343,8 +353,8 @@ __device__ __forceinline__ void gather_quad(const float *xr, const int4 &i1, con
     }
 }
 
-// Stores the slab histogram to w_grad.
-template <int LAYOUT>
+// Stores the slab histogram to w_grad (NT threads).
+template <int LAYOUT, int NT>
 __device__ __forceinline__ void store_slab(const float *hist, float *__restrict__ w_grad, int tid, int m0,
                                            int k0, int rn, int kn, int kc, int log2r, int K, int M,
                                            int vec_out, bool accumulate)
@@ -353,7 +363,7 @@ __device__ __forceinline__ void store_slab(const float *hist, float *__restrict_
     if (accumulate) {
         // the batch is split over several workgroups per slab: w_grad was cleared beforehand and
         // every workgroup adds its share (cells it never touched are skipped)
-        for (int e = tid; e < (LAYOUT == MAM_W_MK ? rn * kn : (kn << log2r)); e += NT_W) {
+        for (int e = tid; e < (LAYOUT == MAM_W_MK ? rn * kn : (kn << log2r)); e += NT) {
             int r, kk;
             float v;
             if (LAYOUT == MAM_W_MK) { r = e / kn; kk = e - r * kn; v = hist[r * kc + kk]; }
@@ -369,19 +379,19 @@ __device__ __forceinline__ void store_slab(const float *hist, float *__restrict_
     if (LAYOUT == MAM_W_MK) {
         if (vec_out) {  // K, k0 and kc are multiples of 4 and w_grad is 16-byte aligned
             const int q = kn >> 2;
-            for (int e = tid; e < rn * q; e += NT_W) {
+            for (int e = tid; e < rn * q; e += NT) {
                 const int r = e / q, c4 = e - r * q;
                 *reinterpret_cast<float4 *>(w_grad + (int64_t)(m0 + r) * K + k0 + c4 * 4) =
                     *reinterpret_cast<const float4 *>(&hist[r * kc + c4 * 4]);
             }
         } else {
-            for (int e = tid; e < rn * kn; e += NT_W) {
+            for (int e = tid; e < rn * kn; e += NT) {
                 const int r = e / kn, kk = e - r * kn;
                 w_grad[(int64_t)(m0 + r) * K + k0 + kk] = hist[r * kc + kk];
             }
         }
     } else {
-        for (int e = tid; e < (kn << log2r); e += NT_W) {
+        for (int e = tid; e < (kn << log2r); e += NT) {
             const int kk = e >> log2r, r = e & (R - 1);
             if (r < rn) w_grad[(int64_t)(k0 + kk) * M + m0 + r] = hist[e];
         }
@@ -394,22 +404,24 @@ __device__ __forceinline__ void store_slab(const float *hist, float *__restrict_
 // the index loads of the next slab are issued before the current slab is streamed out, and the x
 // gathers are in flight while the histogram is cleared, so the scatter phase's latency chain
 // (index load -> gather -> LDS add) overlaps the store phase instead of alternating with it.
-template <int LAYOUT>
-__global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
+// The work of one workgroup (NT threads) of mam_bwd_w_vec_kernel: workgroup `bx` of `nbx` along the slabs,
+// k chunk `by`, share `bz` of `nbz` of the batch rows.
+template <int LAYOUT, int NT>
+__device__ __forceinline__ void bwd_w_vec_body(
+    float *hist, int bx, int nbx, int by, int bz, int nbz,
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
     const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
     int kc, int vec_out, int mtiles, int tiles_per_wg, int rows_per_split, int planes, int range_len)
 {
-    extern __shared__ float hist[];
     const int tid = threadIdx.x;
     const int R = 1 << log2r;
     const int qpr = R >> 2;
-    // blockIdx.z: which share of the batch rows (one share = the whole batch unless the host split it)
-    const int n_begin = blockIdx.z * rows_per_split;
+    // bz: which share of the batch rows (one share = the whole batch unless the host split it)
+    const int n_begin = bz * rows_per_split;
     const int n_rows = (N - n_begin) < rows_per_split ? (N - n_begin) : rows_per_split;
-    const bool accumulate = gridDim.z > 1;
-    const int k0 = blockIdx.y * kc;
+    const bool accumulate = nbz > 1;
+    const int k0 = by * kc;
     const int kn = (K - k0) < kc ? (K - k0) : kc;
     // planes > 1 (the module's `splits`): one (argmax, argmin) pair of absolute k per K range of
     // `range_len`, [plane][N*M]; a slab takes the planes whose ranges meet its k chunk
@@ -419,7 +431,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
     const int npl = pl_hi - pl_lo + 1;
     const int64_t per_plane = (int64_t)n_rows * qpr;
     const int64_t items = per_plane * npl;
-    const int first = xcd_remap(blockIdx.x, gridDim.x) * tiles_per_wg;
+    const int first = xcd_remap(bx, nbx) * tiles_per_wg;
 
     // this thread's first item of a slab: plane pl_lo + pf, row n_first, neurons m0 + r_first .. +3
     const int pf = npl > 1 ? (int)(tid / per_plane) : 0;
@@ -452,11 +464,11 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
         const int rn = (M - m0) < R ? (M - m0) : R;
         float x1[4] = {s1.x, s1.y, s1.z, s1.w}, x2[4] = {s2.x, s2.y, s2.z, s2.w};
         if (have && !x_sel) gather_quad(x + (int64_t)n_first * ldx + k0, i1, i2, k0, kn, x1, x2);
-        for (int i = tid * 4; i < R * kc; i += NT_W * 4)
+        for (int i = tid * 4; i < R * kc; i += NT * 4)
             *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
         if (have) scatter_quad<LAYOUT>(hist, g, i1, i2, x1, x2, r_first, k0, kn, kc, log2r);
-        for (int64_t it = tid + NT_W; it < items; it += NT_W) {
+        for (int64_t it = tid + NT; it < items; it += NT) {
             const int pl = npl > 1 ? (int)(it / per_plane) : 0;
             const int64_t rem = npl > 1 ? it - pl * per_plane : it;
             const int n = n_begin + (int)(rem / qpr), r0 = (int)(rem % qpr) * 4;
@@ -479,8 +491,50 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
         }
         __syncthreads();
         if (t + 1 < tiles_per_wg && mt + 1 < mtiles) load_first(m0 + R);
-        store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, accumulate);
+        store_slab<LAYOUT, NT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, accumulate);
         __syncthreads();
+    }
+}
+
+template <int LAYOUT>
+__global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
+    const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
+    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
+    const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
+    int kc, int vec_out, int mtiles, int tiles_per_wg, int rows_per_split, int planes, int range_len)
+{
+    extern __shared__ float hist[];
+    bwd_w_vec_body<LAYOUT, NT_W>(hist, blockIdx.x, gridDim.x, blockIdx.y, blockIdx.z, gridDim.z, x, ldx, grad, argmax,
+                                 argmin, x_sel, nm, w_grad, N, K, M, log2r, kc, vec_out, mtiles, tiles_per_wg,
+                                 rows_per_split, planes, range_len);
+}
+
+// Both gradients in one launch, for the shapes where one launch of each kind fills the chip once: the first
+// `x_wgs` workgroups are those of mam_bwd_x_kernel (one batch row each), the rest those of
+// mam_bwd_w_vec_kernel with NT_X threads.  Workgroups are dispatched in index order, so every x_grad workgroup
+// is resident before the first w_grad one: x_grad is bound by LDS atomics, w_grad by its stream to HBM, and
+// side by side they take about as long as w_grad alone.  (Dealt out alternately, the long-running w_grad
+// workgroups end up holding every slot.)
+struct BothParams {
+    const float *x, *w, *grad, *w_sel, *x_sel;
+    const int32_t *argmax, *argmin;
+    float *x_grad, *w_grad;
+    int64_t ldx, ldw, nm;
+    int N, K, M, planes, range_len, span, kc_x;
+    int log2r, kc_w, vec_out, mtiles, tiles_per_wg, x_wgs;
+};
+template <int LAYOUT>
+__global__ __launch_bounds__(NT_X) void mam_bwd_both_kernel(const BothParams p)
+{
+    extern __shared__ unsigned long long both_lds[];
+    if ((int)blockIdx.x < p.x_wgs) {
+        bwd_x_body<LAYOUT>(both_lds, blockIdx.x, p.w, p.ldw, p.grad, p.argmax, p.argmin, p.w_sel, p.nm, p.x_grad, p.K,
+                           p.M, p.kc_x, p.planes, p.span);
+    } else {
+        bwd_w_vec_body<LAYOUT, NT_X>(reinterpret_cast<float *>(both_lds), blockIdx.x - p.x_wgs, gridDim.x - p.x_wgs, 0,
+                                     0, 1, p.x, p.ldx, p.grad, p.argmax, p.argmin, p.x_sel, p.nm, p.w_grad, p.N, p.K,
+                                     p.M, p.log2r, p.kc_w, p.vec_out, p.mtiles, p.tiles_per_wg, p.N, p.planes,
+                                     p.range_len);
     }
 }
 
@@ -528,7 +582,7 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_kernel(
         }
     }
     __syncthreads();
-    store_slab<LAYOUT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, false);
+    store_slab<LAYOUT, NT_W>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, false);
 }
 
 // LDS a workgroup may use for a histogram, in floats, per device.  gfx950 has 160 KiB per CU; above
@@ -548,6 +602,7 @@ static int setup_device(int dev)
         (const void *)mam_bwd_x_kernel<MAM_W_MK>,      (const void *)mam_bwd_x_kernel<MAM_W_KM>,
         (const void *)mam_bwd_w_kernel<MAM_W_MK>,      (const void *)mam_bwd_w_kernel<MAM_W_KM>,
         (const void *)mam_bwd_w_vec_kernel<MAM_W_MK>,  (const void *)mam_bwd_w_vec_kernel<MAM_W_KM>,
+        (const void *)mam_bwd_both_kernel<MAM_W_MK>,
     };
     bool all = true;
     for (const void *k : kernels)
@@ -657,6 +712,51 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
     return rc;
 }
 
+// Both gradients in one launch (mam_bwd_both_kernel) where the shape allows it: (M,K) weights, the 16-byte
+// paths of both kernels, a batch small enough that the x_grad workgroups (one per batch row) are all resident
+// at once, K in one chunk of either kernel -- and, unless the option forces it, at most 2^16 outputs.
+// Returns MAM_OK after launching, 1 when the shape is not served.
+static int launch_both(const float *x, int64_t ldx, const float *w, int64_t ldw, const float *grad,
+                       const int32_t *argmax, const int32_t *argmin, const float *w_sel, const float *x_sel,
+                       float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, hipStream_t st, int planes,
+                       int range_len, bool auto_mode)
+{
+    if (planes <= 1) range_len = (int)K;
+    const int dev = ensure_device();
+    if (dev < 0) return dev;
+    const int cus = num_cus();
+    const bool vec_in = (M % 4 == 0) && (N * M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
+                        ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) &&
+                        ((uintptr_t)x_sel % 16 == 0);
+    constexpr int64_t kLds = 64 * 1024;               // dynamic LDS of the launch: two workgroups per CU
+    const int log2r = 2, R = 4;
+    const int64_t kc_w = (K + 3) / 4 * 4;
+    // Worth it only where the launches themselves are what a call costs (config 1: 10 -> 7 us).  At
+    // 256 x 4096 x 4096 one launch took 35.6 us against 29.2 us for two, with one slab or two per w_grad
+    // workgroup: the x_grad workgroups hold one of the two slots of every CU for as long as they run.
+    const bool small = (auto_mode ? N * M <= (1 << 16) : true);
+    if (!small || !vec_in || N >= 2048 || N > 2 * cus || K * 8 > kLds || R * kc_w * 4 > kLds ||
+        g_lds_floats[dev] * 4 < (int)kLds + 8192)
+        return 1;
+    const int64_t mtiles = ceil_div(M, R);
+    int tpw = (int)(mtiles / (2 * cus));
+    if (tpw < 1) tpw = 1;
+    if (tpw > 8) tpw = 8;
+    const int64_t w_wgs = ceil_div(mtiles, tpw);
+    if (N + w_wgs > INT32_MAX) return 1;
+    BothParams p;
+    p.x = x; p.w = w; p.grad = grad; p.w_sel = w_sel; p.x_sel = x_sel;
+    p.argmax = argmax; p.argmin = argmin; p.x_grad = x_grad; p.w_grad = w_grad;
+    p.ldx = ldx; p.ldw = ldw; p.nm = N * M;
+    p.N = (int)N; p.K = (int)K; p.M = (int)M; p.planes = planes; p.range_len = range_len;
+    p.span = window_span(2 * M * planes); p.kc_x = (int)K;
+    p.log2r = log2r; p.kc_w = (int)kc_w; p.vec_out = (K % 4 == 0) && ((uintptr_t)w_grad % 16 == 0);
+    p.mtiles = (int)mtiles; p.tiles_per_wg = tpw; p.x_wgs = (int)N;
+    const size_t lds = (size_t)(K * 8 > R * kc_w * 4 ? K * 8 : R * kc_w * 4);
+    hipLaunchKernelGGL((mam_bwd_both_kernel<MAM_W_MK>), dim3((unsigned)(N + w_wgs)), dim3(NT_X), lds, st, p);
+    return check_launch("mam_bwd_both_kernel");
+}
+
 // x_grad from selected weights handed over by a forward, whatever that forward read them from.
 int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t *argmin, const float *w_sel,
                          float *x_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
@@ -703,7 +803,15 @@ static int backward_impl(const float *x, int64_t ldx, const float *w, int64_t ld
         return bwd::launch_layout<MAM_W_KM>(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, xg, wg, N, K, M, on,
                                             planes, range_len);
     };
-    // x_grad is bound by LDS atomics and w_grad by memory traffic, and neither depends on the other
+    // x_grad is bound by LDS atomics and w_grad by memory traffic, and neither depends on the other: one
+    // launch that holds both where the shape allows it, else two streams where that pays
+    if (x_grad && w_grad && w_layout == MAM_W_MK && option(MAM_OPT_BACKWARD_ONE_LAUNCH) != MAM_BACKWARD_ONE_LAUNCH_OFF &&
+        option(MAM_OPT_BACKWARD_FORK) != MAM_BACKWARD_FORK_ON) {
+        const int rc = bwd::launch_both(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, x_grad, w_grad, N, K, M, st,
+                                        planes, range_len,
+                                        option(MAM_OPT_BACKWARD_ONE_LAUNCH) == MAM_BACKWARD_ONE_LAUNCH_AUTO);
+        if (rc != 1) return rc;
+    }
     if (x_grad && w_grad) {
         ForkedStream fork(st, N * M);
         if (fork.forked()) {

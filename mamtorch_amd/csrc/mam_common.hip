@@ -129,6 +129,7 @@ int env_choice(const char *name, int fallback)
 std::atomic<int> g_options[MAM_OPT_COUNT_] = {
     {env_choice("MAM_FORWARD_TILING", MAM_FORWARD_TILING_AUTO)},
     {env_choice("MAM_BACKWARD_FORK", MAM_BACKWARD_FORK_AUTO)},
+    {env_choice("MAM_BACKWARD_ONE_LAUNCH", MAM_BACKWARD_ONE_LAUNCH_AUTO)},
 };
 }  // namespace
 

@@ -39,9 +39,6 @@ __device__ __forceinline__ bool fixed_add(unsigned long long *cell, float t, int
     const uint32_t sh = ((b >> 23) & 0xffu) - (uint32_t)e_lo;
     if (sh < (uint32_t)span) {
         const unsigned long long mag = (unsigned long long)((b & 0x7fffffu) | 0x800000u) << sh;
-#ifdef MAM_EXP_NOATOMIC
-        if (mag == 12345ull)
-#endif
         __hip_atomic_fetch_add(cell, (b >> 31) ? 0ull - mag : mag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         return false;
     }

@@ -237,6 +237,34 @@ def test_x_grad_on_the_second_stream_or_not(fork):
         capi.set_option(capi.OPT_BACKWARD_FORK, capi.BACKWARD_FORK_AUTO)
 
 
+@pytest.mark.parametrize("shape", [(64, 784, 256), (96, 200, 64), (256, 1024, 512), (130, 4096, 72), (40, 36, 8)])
+def test_both_gradients_in_one_launch_or_two(shape):
+    """(M,K) weights, aligned operands, a batch below twice the CU count, K <= 4096: one launch can hold the
+    workgroups of both gradient kernels (option MAM_OPT_BACKWARD_ONE_LAUNCH: by default for small calls, 2 =
+    wherever the shape allows it, 0 = never).  Either way the
+    results meet the oracle; x_grad from handed-over weights is the exact sum, so the two ways agree bit for bit."""
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    N, K, M = shape
+    x, w, grad = random_case(N, K, M, seed=N + M)
+    _, amax, amin = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+    got = {}
+    try:
+        for mode in (0, 2):
+            capi.set_option(capi.OPT_BACKWARD_ONE_LAUNCH, mode)
+            _check(x, w, grad, amax, amin, "one launch=%d shape %s" % (mode, shape), layouts=(capi.W_MK,))
+            w_sel = torch.empty(2, N, M, device=dev)
+            x_sel = torch.empty(2, N, M, device=dev)
+            c, a1, a2 = capi.fc_forward(x.to(dev), w.to(dev), capi.W_MK, w_sel=w_sel, x_sel=x_sel)
+            got[mode] = capi.fc_backward(x.to(dev), w.to(dev), grad.to(dev), a1, a2, capi.W_MK, w_sel=w_sel, x_sel=x_sel)
+            torch.cuda.synchronize()
+    finally:
+        capi.set_option(capi.OPT_BACKWARD_ONE_LAUNCH, 1)
+    assert torch.equal(got[0][0].view(torch.int32), got[2][0].view(torch.int32)), "x_grad differs between the two ways"
+    # w_grad: two orders of fp32 additions, each held to the oracle's bar by _check above
+
+
 def _dynamic_range_grad(N, M, pattern, seed):
     """grad whose terms span far more binades than a 64-bit fixed-point window holds."""
     g = torch.Generator().manual_seed(seed)
