@@ -51,6 +51,15 @@ def test_argument_validation_without_a_gpu():
     assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, None, 2, 4, 2, None, 0, None) == -1
     assert b"null" in l.mam_last_error()
     assert l.mam_selection_count(None, None, None, None, 2, 2, 2, 9, None) == -1
+    # sizes beyond what the kernels index are refused, not truncated (pointers never dereferenced)
+    one = ctypes.c_void_p(16)
+    big = 2 ** 30 + 1
+    assert l.mam_fc_forward(one, big, one, big, 0, None, one, one, one, None, None, 2, big, 2, None, 0, None) == -2
+    assert b"2^30" in l.mam_last_error()
+    assert l.mam_fc_backward(one, 4, one, 4, 1, one, one, one, None, None, one, one, big, 4, 2, None) == -2
+    assert l.mam_selection_count(one, one, one, one, 2, big, 2, 1, None) == -2
+    assert l.mam_fc_forward(one, 2, one, 4, 0, None, one, one, one, None, None, 2, 4, 2, None, 0, None) == -1
+    assert b"leading dimension" in l.mam_last_error()
     # empty problems are a no-op
     assert l.mam_fc_forward(None, 4, None, 4, 0, None, None, None, None, None, None, 0, 4, 2, None, 0, None) == 0
     assert l.mam_selection_count(None, None, None, None, 0, 2, 2, 0, None) == 0

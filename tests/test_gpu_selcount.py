@@ -54,6 +54,29 @@ def test_random_indices(shape, mode):
         assert int(got[0].sum() - mc.sum()) == N * M and int(got[1].sum() - nc.sum()) == N * M
 
 
+@pytest.mark.parametrize("M", [4, 5])
+def test_more_hits_on_one_cell_than_a_16_bit_field_holds(M):
+    """Hits mode counts in 16-bit LDS fields; batches above 32768 rows are walked in passes so that a field
+    cannot overflow.  70000 rows that all pick the same weight must add exactly 70000 (both the 16-byte path,
+    M a multiple of 4, and the element path)."""
+    N, K = 70000, 8
+    amax = np.full((N, M), 3, np.int32)
+    amin = np.full((N, M), 5, np.int32)
+    amin[:, 0] = 3                      # one neuron picks the same weight as max and as min
+    z = np.zeros((M, K), np.int32)
+    for mode in (1, 0, 2):
+        mc, nc = _run(amax, amin, z, z, mode)
+        want = oracle.selection_count(amax, amin, z, z, mode) if mode != 2 else None
+        if mode == 1:
+            assert mc[:, 3].tolist() == [N] * M and nc[1:, 5].tolist() == [N] * (M - 1) and nc[0, 3] == N
+            assert int(mc.sum()) == N * M and int(nc.sum()) == N * M
+        if want is not None:
+            np.testing.assert_array_equal(mc, want[0])
+            np.testing.assert_array_equal(nc, want[1])
+        if mode == 2:                   # flags, max and min apart: one per picked cell
+            assert int(mc.sum()) == M and int(nc.sum()) == M and mc[0, 3] == 1 and nc[0, 3] == 1
+
+
 def test_headline_config2_accumulates_over_batches():
     from mamtorch_amd import capi
 
