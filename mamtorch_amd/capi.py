@@ -160,6 +160,15 @@ def set_option(option, value):
     _check(lib().mam_set_option(option, value))
 
 
+def fc_forward_describe(x, w, layout=W_KM, with_indices=True):
+    """Text naming the kernels and the tiling that mam_fc_forward would launch for these operands."""
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    buf = ctypes.create_string_buffer(320)
+    _check(l.mam_fc_forward_describe(_p(x), _ld(x), _p(w), _ld(w), layout, N, K, M, 1 if with_indices else 0, buf, 320))
+    return buf.value.decode()
+
+
 def fc_forward_values(x, w, layout=W_KM, bias=None, workspace=None):
     l = lib()
     N, K, M = _dims(x, w, layout)

@@ -69,6 +69,7 @@ struct Params {
     int vec_x, vec_w;  // 16-byte global loads are legal for x / w
     int fast;          // the k-invariant 32-bit-offset staging path is legal
     int coop;          // the cooperative resolve is legal: (M,K) w, 16-byte rows, K % G == 0
+    int gt;            // products per recorded group: G, or 2 G on the wave-uniform-rows tiling at large K
 };
 
 // First k in group g (ascending) whose product equals `target`; value recomputed from it.
@@ -190,53 +191,72 @@ __device__ __forceinline__ int quad_min(int v)
     return o < v ? o : v;
 }
 
-//   operands(r, slot, sub, kb, xp, wp): where the 4 x and 4 w operands k = kb .. kb+3 of the task in round r
-//   live.  The addresses are most of the instructions of a round when they are formed in 64 bits per
+//   operands(r, slot, sub, kb, xp, wp): where the GT/4 x and GT/4 w operands k = kb .. kb+GT/4-1 of the task in
+//   round r live.  The addresses are most of the instructions of a round when they are formed in 64 bits per
 //   lane, so a caller whose 64 outputs share bases hands in something cheaper.
-template <class NM, class OP>
+//   GT: the k loop's tracking span, 16 or 32 products per recorded group; a lane takes GT/4 of them (one or two
+//   16-byte loads per operand), and the loads of 8 * 16 / GT rounds are in flight together.
+template <int GT, class NM, class OP>
 __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps, float *res,
                                              int lane, NM nm_of, OP operands)
 {
+    static_assert(GT == 16 || GT == 32, "tracking span");
+    constexpr int PPL = GT / LPT;             // products per lane
+    constexpr int NV = PPL / 4;               // 16-byte loads per operand and lane
+    constexpr int BATCH = RES_ROUNDS / NV;    // rounds whose loads are issued before the first use
     float *res_v = res;                                    // [2][64]
     int *res_i = reinterpret_cast<int *>(res + 128);        // [2][64]
     float *res_w = res + 256;                               // [2][64]
     float *res_x = res + 384;                               // [2][64]
-    // every load of every round first, then the matching
-    float4 xa[RES_ROUNDS], wa[RES_ROUNDS];
-    float target[RES_ROUNDS];
-    int grp[RES_ROUNDS];
 #pragma unroll
-    for (int r = 0; r < RES_ROUNDS; ++r) {
-        const int task = r * TPR + lane / LPT;
-        const int slot = task >> 1, ext = task & 1, sub = lane % LPT;
-        target[r] = vals[ext * 64 + slot];
-        grp[r] = grps[ext * 64 + slot];
-        const float *xp, *wp;
-        operands(r, slot, sub, grp[r] * G + sub * 4, xp, wp);
-        xa[r] = *reinterpret_cast<const float4 *>(xp);
-        wa[r] = *reinterpret_cast<const float4 *>(wp);
-    }
+    for (int r0 = 0; r0 < RES_ROUNDS; r0 += BATCH) {
+        // every load of the batch first, then the matching
+        float4 xa[BATCH][NV], wa[BATCH][NV];
+        float target[BATCH];
+        int grp[BATCH];
 #pragma unroll
-    for (int r = 0; r < RES_ROUNDS; ++r) {
-        const int task = r * TPR + lane / LPT;
-        const int slot = task >> 1, ext = task & 1, sub = lane % LPT;
-        const float p0 = xa[r].x * wa[r].x, p1 = xa[r].y * wa[r].y, p2 = xa[r].z * wa[r].z, p3 = xa[r].w * wa[r].w;
-        // position within the group of this lane's first match (lowest wins), 255 = none
-        int key = 255;
-        float wsel = wa[r].x, xsel = xa[r].x;      // kept only by the fallback below
-        if (p3 == target[r]) { key = sub * 4 + 3; wsel = wa[r].w; xsel = xa[r].w; }
-        if (p2 == target[r]) { key = sub * 4 + 2; wsel = wa[r].z; xsel = xa[r].z; }
-        if (p1 == target[r]) { key = sub * 4 + 1; wsel = wa[r].y; xsel = xa[r].y; }
-        if (p0 == target[r]) { key = sub * 4 + 0; wsel = wa[r].x; xsel = xa[r].x; }
-        const int best = quad_min(key);
-        // no product equals the extreme (NaN operands): the first k of the group, from lane 0
-        const bool fallback = best == 255 && sub == 0;
-        if ((key == best && key != 255) || fallback) {
-            // the value is recomputed from the selected operands (the sign of a zero follows them)
-            res_v[ext * 64 + slot] = fallback ? target[r] : xsel * wsel;
-            res_i[ext * 64 + slot] = grp[r] * G + (fallback ? 0 : key);
-            res_w[ext * 64 + slot] = wsel;
-            res_x[ext * 64 + slot] = xsel;
+        for (int b = 0; b < BATCH; ++b) {
+            const int r = r0 + b;
+            const int task = r * TPR + lane / LPT;
+            const int slot = task >> 1, ext = task & 1, sub = lane % LPT;
+            target[b] = vals[ext * 64 + slot];
+            grp[b] = grps[ext * 64 + slot];
+            const float *xp, *wp;
+            operands(r, slot, sub, grp[b] * GT + sub * PPL, xp, wp);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                xa[b][v] = reinterpret_cast<const float4 *>(xp)[v];
+                wa[b][v] = reinterpret_cast<const float4 *>(wp)[v];
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) {
+            const int r = r0 + b;
+            const int task = r * TPR + lane / LPT;
+            const int slot = task >> 1, ext = task & 1, sub = lane % LPT;
+            // position within the group of this lane's first match (lowest wins), 255 = none
+            int key = 255;
+            float wsel = wa[b][0].x, xsel = xa[b][0].x;      // kept only by the fallback below
+#pragma unroll
+            for (int v = NV - 1; v >= 0; --v) {
+                const float p0 = xa[b][v].x * wa[b][v].x, p1 = xa[b][v].y * wa[b][v].y, p2 = xa[b][v].z * wa[b][v].z,
+                            p3 = xa[b][v].w * wa[b][v].w;
+                const int k0 = sub * PPL + v * 4;
+                if (p3 == target[b]) { key = k0 + 3; wsel = wa[b][v].w; xsel = xa[b][v].w; }
+                if (p2 == target[b]) { key = k0 + 2; wsel = wa[b][v].z; xsel = xa[b][v].z; }
+                if (p1 == target[b]) { key = k0 + 1; wsel = wa[b][v].y; xsel = xa[b][v].y; }
+                if (p0 == target[b]) { key = k0 + 0; wsel = wa[b][v].x; xsel = xa[b][v].x; }
+            }
+            const int best = quad_min(key);
+            // no product equals the extreme (NaN operands): the first k of the group, from lane 0
+            const bool fallback = best == 255 && sub == 0;
+            if ((key == best && key != 255) || fallback) {
+                // the value is recomputed from the selected operands (the sign of a zero follows them)
+                res_v[ext * 64 + slot] = fallback ? target[b] : xsel * wsel;
+                res_i[ext * 64 + slot] = grp[b] * GT + (fallback ? 0 : key);
+                res_w[ext * 64 + slot] = wsel;
+                res_x[ext * 64 + slot] = xsel;
+            }
         }
     }
     // lane s finishes output s
@@ -266,7 +286,7 @@ template <class NM>
 __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals, const int *grps, float *res,
                                              int lane, NM nm_of)
 {
-    resolve_wave(p, vals, grps, res, lane, nm_of,
+    resolve_wave<G>(p, vals, grps, res, lane, nm_of,
                  [&](int, int slot, int, int kb, const float *&xp, const float *&wp) {
                      int n, m;
                      bool valid;
@@ -647,7 +667,7 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 
 // Combines split-K partials in ascending k order (strict comparisons keep the earliest
 // group on ties), then resolves indices / zero signs exactly as the single-pass epilogue.
-template <int LAYOUT, bool ARGS, bool COOP>
+template <int LAYOUT, bool ARGS, bool COOP, int GT = G>
 __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
 {
     // A workgroup owns a 16 x 16 patch of c.  Resolving re-reads G weights of row m per output,
@@ -664,7 +684,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
     const bool live = n_own < p.N && m_own < p.M;
     const int64_t o = (int64_t)n_own * p.M + m_own;
     const int stride = ARGS ? 3 : 2;
-    const int gps = p.k_per_split / G;   // groups per split
+    const int gps = p.k_per_split / GT;   // groups per split
     float vmax = 0.0f, vmin = 0.0f;
     int gmax = 0, gmin = 0;
     if (live) {
@@ -707,7 +727,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
         const uint32_t ldw4 = (uint32_t)p.ldw * 4u;
         const uint32_t last = last_row_offset(p.M, mb, 16, ldw4);
         const uint32_t mine = (uint32_t)(lane >> 3) * ldw4;
-        resolve_wave(p, &vals_s[wave][0][0], &grps_s[wave][0][0], &res_s[wave][0], lane,
+        resolve_wave<GT>(p, &vals_s[wave][0][0], &grps_s[wave][0][0], &res_s[wave][0], lane,
                      [&](int slot, int &n, int &m, bool &valid) {
                          n = nbase + (slot >> 4);
                          m = mbase + (slot & 15);
@@ -724,6 +744,7 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
                          wp = reinterpret_cast<const float *>(wrows + (clamped_row_offset(row, last) + k4));
                      });
     } else if (live) {
+        static_assert(COOP || GT == G, "the per-thread resolve scans groups of G");
         finish<LAYOUT, ARGS>(p, n_own, m_own, vmax, vmin, gmax, gmin);
     }
 }
@@ -821,7 +842,11 @@ typedef const __attribute__((address_space(4))) float const_f32;
 
 // TAIL: K (or the last K range) is a multiple of G = 16 but not of 64; the last tile is partial.  A separate
 // instantiation, so that the whole-tile kernel stays exactly what it was.
-template <int TJ, bool ARGS, bool SPLIT, bool TAIL>
+// GT: products per recorded group.  G = 16 costs a compare and a select per extreme and 16 products; with
+// GT = 32 the pair is issued after every second group (the running extremes of the first are kept as the
+// baseline), which takes 64 of a tile's 1160 instructions off the k loop and doubles what the resolve scans
+// per output: taken where the resolve is cheap next to the loop (K >= 2048), whole 64-k tiles only.
+template <int TJ, bool ARGS, bool SPLIT, bool TAIL, int GT = G>
 __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 {
     using C = sx::Cfg<TJ>;
@@ -848,7 +873,9 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     const int ke = (kb + p.k_per_split) < p.K ? (kb + p.k_per_split) : p.K;
     const int ntiles = (ke - kb) / sx::KT;    // whole tiles; a rest of whole 16-k groups follows as a partial tile
 
+    static_assert(GT == G || (GT == 2 * G && !TAIL), "tracking span");
     float vmax[sx::TI][TJ], vmin[sx::TI][TJ];
+    float bmax[sx::TI][TJ], bmin[sx::TI][TJ];     // GT > G: the extremes before the first group of a span
     int gmax[sx::TI][TJ], gmin[sx::TI][TJ];
 #pragma unroll
     for (int i = 0; i < sx::TI; ++i)
@@ -856,6 +883,8 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
         for (int j = 0; j < TJ; ++j) {
             vmax[i][j] = -__builtin_inff();
             vmin[i][j] = __builtin_inff();
+            bmax[i][j] = vmax[i][j];
+            bmin[i][j] = vmin[i][j];
             gmax[i][j] = 0;
             gmin[i][j] = 0;
         }
@@ -906,7 +935,8 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
 #pragma unroll
         for (int gg = 0; gg < sx::KT / G; ++gg) {
             if (TAIL && gg >= ng) break;
-            const int grel = t * (sx::KT / G) + gg;
+            const int grel = (t * sx::KT + gg * G) / GT;       // the span this group belongs to
+            const bool opens = (gg * G) % GT == 0, closes = ((gg + 1) * G) % GT == 0;
             float xv[sx::TI][G];
 #pragma unroll
             for (int i = 0; i < sx::TI; ++i)
@@ -923,15 +953,16 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
                 }
 #pragma unroll
                 for (int i = 0; i < sx::TI; ++i) {
-                    const float om = vmax[i][j], on = vmin[i][j];
-                    float hi = om, lo = on;
+                    if (GT > G && opens) { bmax[i][j] = vmax[i][j]; bmin[i][j] = vmin[i][j]; }
+                    const float om = GT > G ? bmax[i][j] : vmax[i][j], on = GT > G ? bmin[i][j] : vmin[i][j];
+                    float hi = vmax[i][j], lo = vmin[i][j];
 #pragma unroll
                     for (int q = 0; q < G; q += 2) {
                         const float a = xv[i][q] * wv[q], b = xv[i][q + 1] * wv[q + 1];
                         hi = __builtin_fmaxf(__builtin_fmaxf(hi, a), b);
                         lo = __builtin_fminf(__builtin_fminf(lo, a), b);
                     }
-                    if (ARGS) {
+                    if (ARGS && closes) {
                         gmax[i][j] = (hi > om) ? grel : gmax[i][j];
                         gmin[i][j] = (lo < on) ? grel : gmin[i][j];
                     }
@@ -977,7 +1008,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     }
 
     // ---- epilogue ----
-    const int g0 = kb / G;
+    const int g0 = kb / GT;
     if (SPLIT) {
         const int64_t nm = (int64_t)p.N * p.M;
         float *base = p.part + (int64_t)split * (ARGS ? 3 : 2) * nm;
@@ -1028,7 +1059,7 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
                 const char *wrows = reinterpret_cast<const char *>(p.w + (int64_t)mb * p.ldw);
                 const uint32_t last = last_row_offset(p.M, mb, 64, ldw4);   // neurons past M repeat the last one
                 const uint32_t mine = (uint32_t)(lane >> 3) * ldw4;         // slot = 8 r + lane / 8
-                resolve_wave(p, vals + j * 128, grps + j * 128, res, lane,
+                resolve_wave<GT>(p, vals + j * 128, grps + j * 128, res, lane,
                              [&](int slot, int &n, int &m, bool &valid) {
                                  n = nrow;
                                  m = mbase + slot;
@@ -1185,6 +1216,8 @@ static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const f
              (p.k_per_split % 4 == 0);
     // (16 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
     p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 25));
+    // two groups per recorded span where the resolve is cheap next to the k loop (see mam_fwd_sx_kernel)
+    p.gt = (args && use_sx && range_len == 0 && K >= 2048 && K % sx::KT == 0 && p.k_per_split % sx::KT == 0) ? 2 * G : G;
     // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
     if ((int64_t)p.k_per_split / G > 65536)
         return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds %d per K range", (long long)K, 65536 * G);
@@ -1267,10 +1300,14 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
     const bool tail = K % sx::KT != 0;
     if (use_sx && p.splits > 1 && tail)
         hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+    else if (use_sx && p.splits > 1 && ARGS && p.gt == 2 * G)
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true, false, ARGS ? 2 * G : G>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (use_sx && p.splits > 1)
         hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, true, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (use_sx && tail)
         hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, false, true>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
+    else if (use_sx && ARGS && p.gt == 2 * G)
+        hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, false, false, ARGS ? 2 * G : G>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (use_sx)
         hipLaunchKernelGGL((mam_fwd_sx_kernel<2, ARGS, false, false>), dim3((unsigned)nblk), dim3(sx::NT), 0, st, p);
     else if (w_layout == MAM_W_MK)
@@ -1289,7 +1326,9 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
         rc = check_launch("mam_fwd_range_sum_kernel");
     } else if (p.splits > 1) {
         const unsigned mb = (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
-        if (ARGS && p.coop)
+        if (ARGS && p.coop && p.gt == 2 * G)
+            hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS, ARGS, ARGS ? 2 * G : G>), dim3(mb), dim3(256), 0, st, p);
+        else if (ARGS && p.coop)
             hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS, ARGS>), dim3(mb), dim3(256), 0, st, p);
         else if (w_layout == MAM_W_MK)
             hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS, false>), dim3(mb), dim3(256), 0, st, p);
@@ -1363,8 +1402,9 @@ extern "C" int mam_fc_forward_describe(const float *x, int64_t ldx, const float 
     const fwd::Params &p = plan.p;
     const char *what = with_indices ? "args" : "values";
     if (plan.use_sx)
-        snprintf(text, text_bytes, "mam_fwd_sx_kernel<%s%s%s> %d x %d tiles of 32 x 128", what, p.splits > 1 ? ", split" : "",
-                 K % fwd::sx::KT != 0 ? ", partial last k tile" : "", p.tiles_n, p.tiles_m);
+        snprintf(text, text_bytes, "mam_fwd_sx_kernel<%s%s%s%s> %d x %d tiles of 32 x 128", what, p.splits > 1 ? ", split" : "",
+                 K % fwd::sx::KT != 0 ? ", partial last k tile" : "", p.gt > fwd::G ? ", indices per 32 k" : "", p.tiles_n,
+                 p.tiles_m);
     else
         snprintf(text, text_bytes, "mam_fwd_kernel<%s, %s> %d x %d tiles of 64 x 128", w_layout == MAM_W_MK ? "(M,K)" : "(K,M)",
                  what, p.tiles_n, p.tiles_m);

@@ -315,6 +315,51 @@ def test_vit_mlp_config3_shapes(dims):
     assert torch.equal(c2, c[perm]) and torch.equal(amax2, amax[perm]) and torch.equal(amin2, amin[perm])
 
 
+@pytest.mark.parametrize("shape", [(64, 2048, 256), (40, 2112, 72), (256, 4096, 128), (2048, 2048, 1024), (2080, 2240, 1000)])
+@pytest.mark.parametrize("data", ["ties", "plain", "zeros"])
+def test_indices_recorded_per_32_products(shape, data):
+    """From K = 2048 on (whole 64-k tiles) the wave-uniform-rows tiling records the group of an extreme once per
+    32 products instead of 16, and the resolve scans 32: the small shapes take the K split and the merge kernel,
+    the large ones the kernel's own epilogue.  Quantised operands make most products tie, also across the two
+    halves of a span and across spans; the first index must still win.  Oracle on a sample of the rows, the
+    selected products reproduce c on all of them, and the general tiling (groups of 16) agrees bit for bit."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    N, K, M = shape
+    g = torch.Generator().manual_seed(N + K + M)
+    x = torch.randn(N, K, generator=g)
+    w = torch.randn(M, K, generator=g)
+    if data == "ties":
+        x, w = torch.round(x), torch.round(w * 2) / 2
+    elif data == "zeros":                       # extremes that are zeros of either sign
+        x = torch.where(torch.rand(N, K, generator=g) < 0.5, torch.zeros(()), -x.abs())
+        w = torch.where(torch.rand(M, K, generator=g) < 0.5, -torch.zeros(()), w.abs())
+    xd, wd = x.to(dev), w.to(dev)
+    text = capi.fc_forward_describe(xd, wd, capi.W_MK)
+    assert "indices per 32 k" in text, text
+    w_sel = torch.empty(2, N, M, device=dev)
+    x_sel = torch.empty(2, N, M, device=dev)
+    c, amax, amin = capi.fc_forward(xd, wd, capi.W_MK, w_sel=w_sel, x_sel=x_sel)
+    cv = capi.fc_forward_values(xd, wd, capi.W_MK)
+    torch.cuda.synchronize()
+    rows = torch.arange(0, N, max(1, N // 48))
+    want = oracle.forward(x[rows].numpy(), w.numpy(), oracle.W_MK)
+    assert_bits_equal(c[rows.to(dev)].cpu().numpy(), want[0], "c")
+    assert_index_equal(amax[rows.to(dev)].cpu().numpy(), want[1], "argmax")
+    assert_index_equal(amin[rows.to(dev)].cpu().numpy(), want[2], "argmin")
+    assert torch.equal(c.view(torch.int32), cv.view(torch.int32))
+    cols = torch.arange(M, device=dev)[None, :]
+    assert torch.equal(w_sel[0], wd[cols, amax.long()]) and torch.equal(w_sel[1], wd[cols, amin.long()])
+    assert torch.equal(x_sel[0], torch.gather(xd, 1, amax.long())) and torch.equal(x_sel[1], torch.gather(xd, 1, amin.long()))
+    assert torch.equal((w_sel[0] * x_sel[0] + w_sel[1] * x_sel[1]).view(torch.int32), c.view(torch.int32))
+    with forward_tiling("wide"):
+        c2, amax2, amin2 = capi.fc_forward(xd, wd, capi.W_MK)
+        torch.cuda.synchronize()
+    assert torch.equal(c2.view(torch.int32), c.view(torch.int32))
+    assert torch.equal(amax2, amax) and torch.equal(amin2, amin)
+
+
 @pytest.mark.parametrize("M", [1024, 4096])
 def test_large_batch_inference_config4(M):
     """N16384 K4096, x~U(-1,1), W~N(0,0.02): oracle on sampled rows + properties on all."""
