@@ -48,7 +48,7 @@ extern "C" {
                                  likewise for min (the retired convolution modules' literal rule)        */
 
 /* Run-time switches for mam_set_option().  Their initial values come from the environment variables of
- * the same names (MAM_FORWARD_TILING = auto | wide, MAM_BACKWARD_FORK = 0 | 1, MAM_BACKWARD_ONE_LAUNCH = 0 | 1), read once when the
+ * the same names (MAM_FORWARD_TILING = auto | wide | 2, MAM_BACKWARD_FORK = 0 | 1, MAM_BACKWARD_ONE_LAUNCH = 0 | 1), read once when the
  * library is loaded. */
 #define MAM_OPT_FORWARD_TILING 0 /* which dense forward tiling serves a call                      */
 #define MAM_OPT_BACKWARD_FORK 1  /* x_grad on the library's second stream beside w_grad           */
@@ -56,6 +56,7 @@ extern "C" {
 #define MAM_OPT_COUNT_ 3
 #define MAM_FORWARD_TILING_AUTO 0 /* wave-uniform-rows tiling where the layout allows it           */
 #define MAM_FORWARD_TILING_WIDE 1 /* every call on the general 64 x 128 tiling                     */
+#define MAM_FORWARD_TILING_GROUPS16 2 /* as AUTO, but indices recorded per 16 products at every K   */
 #define MAM_BACKWARD_FORK_AUTO (-1) /* from 2^22 outputs on, and under stream capture from 2^16   */
 #define MAM_BACKWARD_FORK_OFF 0
 #define MAM_BACKWARD_FORK_ON 1

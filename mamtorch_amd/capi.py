@@ -20,6 +20,7 @@ OPT_BACKWARD_FORK = 1
 OPT_BACKWARD_ONE_LAUNCH = 2
 FORWARD_TILING_AUTO = 0
 FORWARD_TILING_WIDE = 1
+FORWARD_TILING_GROUPS16 = 2
 BACKWARD_FORK_AUTO = -1
 COUNT_REFERENCE = 0
 COUNT_HITS = 1

@@ -1217,7 +1217,8 @@ static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const f
     // (16 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
     p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 25));
     // two groups per recorded span where the resolve is cheap next to the k loop (see mam_fwd_sx_kernel)
-    p.gt = (args && use_sx && range_len == 0 && K >= 2048 && K % sx::KT == 0 && p.k_per_split % sx::KT == 0) ? 2 * G : G;
+    p.gt = (args && use_sx && range_len == 0 && K >= 2048 && K % sx::KT == 0 && p.k_per_split % sx::KT == 0 &&
+            option(MAM_OPT_FORWARD_TILING) != MAM_FORWARD_TILING_GROUPS16) ? 2 * G : G;
     // group ids are kept as 16-bit offsets from the first group of a workgroup's k range
     if ((int64_t)p.k_per_split / G > 65536)
         return fail(MAM_ERR_UNSUPPORTED, "K = %lld exceeds %d per K range", (long long)K, 65536 * G);
