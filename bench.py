@@ -82,8 +82,8 @@ class Layer:
         if want_count:
             self.max_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
             self.min_count = torch.zeros((M, K), dtype=torch.int32, device=dev)
-        query = lib.mam_fc_forward_values_workspace if values_only else lib.mam_fc_forward_workspace
-        self.ws_bytes = query(N, K, M)
+        # what the operators and capi bring: the required bytes plus the optional room the library can use
+        self.ws_bytes = lib.mam_fc_forward_workspace_for(N, K, M, capi.W_MK, 0 if values_only else 1)
         self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
         self.torch, self.dev = torch, dev
 
