@@ -670,17 +670,20 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
 template <int LAYOUT, bool ARGS, bool COOP, int GT = G>
 __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
 {
-    // A workgroup owns a 16 x 16 patch of c.  Resolving re-reads G weights of row m per output,
-    // i.e. random lines of the weight matrix; ordering the patches so that all batch patches of
-    // one 16-neuron range run back to back on one XCD keeps those 16 weight rows in that L2.
+    // A workgroup owns a PR x PC patch of c (16 x 16; with the cooperative resolve 4 x 64: a wave takes one batch
+    // row, and its piece of every partial plane and of every output array is two whole 128-byte lines; measured at
+    // 256 x 4096 x 4096: 28.4 us with 16 x 16, 27.0 with 8 x 32, 26.6 with 4 x 64).  Resolving re-reads GT
+    // weights of row m per output, i.e. random lines of the weight matrix; ordering the patches so that all batch
+    // patches of one PC-neuron range run back to back on one XCD keeps those weight rows in that L2.
+    constexpr int PC = COOP ? 64 : 16, PR = 256 / PC, LOG2PC = COOP ? 6 : 4;
     __shared__ float vals_s[4][2][64];
     __shared__ int grps_s[4][2][64];
     __shared__ float res_s[4][RES_WORDS];
     const int64_t nm = (int64_t)p.N * p.M;
-    const int patches_n = (p.N + 15) / 16;
+    const int patches_n = (p.N + PR - 1) / PR;
     const int logical = xcd_remap(blockIdx.x, gridDim.x);
     const int pm = logical / patches_n, pn = logical - pm * patches_n;
-    const int n_own = pn * 16 + (threadIdx.x >> 4), m_own = pm * 16 + (threadIdx.x & 15);
+    const int n_own = pn * PR + (threadIdx.x >> LOG2PC), m_own = pm * PC + (threadIdx.x & (PC - 1));
     const bool live = n_own < p.N && m_own < p.M;
     const int64_t o = (int64_t)n_own * p.M + m_own;
     const int stride = ARGS ? 3 : 2;
@@ -718,27 +721,28 @@ __global__ __launch_bounds__(256) void mam_fwd_merge_kernel(const Params p)
         grps_s[wave][0][lane] = gmax;
         grps_s[wave][1][lane] = gmin;
         __syncthreads();
-        const int nbase = pn * 16 + 4 * wave, mbase = pm * 16;
-        // slot = 8 r + lane / 8 in round r: batch row nbase + r / 2 (the same for the whole wave) and
-        // neuron mbase + 8 (r & 1) + lane / 8, so the operands sit at 32-bit byte offsets from
-        // wave-uniform bases (the host checked that 16 rows of w span < 4 GiB)
+        const int nbase = pn * PR + (PR / 4) * wave, mbase = pm * PC;
+        // slot = 8 r + lane / 8 in round r: batch row nbase + slot / PC (the same for the whole wave) and
+        // neuron mbase + slot % PC = mbase + 8 (r % (PC / 8)) + lane / 8, so the operands sit at 32-bit byte
+        // offsets from wave-uniform bases (the host checked that PC rows of w span < 4 GiB)
         const int mb = mbase < p.M ? mbase : p.M - 1;
         const char *wrows = reinterpret_cast<const char *>(p.w + (int64_t)mb * p.ldw);
         const uint32_t ldw4 = (uint32_t)p.ldw * 4u;
-        const uint32_t last = last_row_offset(p.M, mb, 16, ldw4);
+        const uint32_t last = last_row_offset(p.M, mb, PC, ldw4);
         const uint32_t mine = (uint32_t)(lane >> 3) * ldw4;
         resolve_wave<GT>(p, &vals_s[wave][0][0], &grps_s[wave][0][0], &res_s[wave][0], lane,
                      [&](int slot, int &n, int &m, bool &valid) {
-                         n = nbase + (slot >> 4);
-                         m = mbase + (slot & 15);
+                         n = nbase + (slot >> LOG2PC);
+                         m = mbase + (slot & (PC - 1));
                          valid = n < p.N && m < p.M;
                          n = n < p.N ? n : p.N - 1;
                          m = m < p.M ? m : p.M - 1;
                      },
                      [&](int r, int, int, int kb, const float *&xp, const float *&wp) {
-                         const int n = (nbase + (r >> 1)) < p.N ? (nbase + (r >> 1)) : (p.N - 1);
+                         const int nr = nbase + (r >> (LOG2PC - 3));
+                         const int n = nr < p.N ? nr : (p.N - 1);
                          const char *xrow = reinterpret_cast<const char *>(p.x + (int64_t)n * p.ldx);
-                         const uint32_t row = mine + (uint32_t)(8 * (r & 1)) * ldw4;
+                         const uint32_t row = mine + (uint32_t)(8 * (r & (PC / 8 - 1))) * ldw4;
                          const uint32_t k4 = (uint32_t)kb * 4u;
                          xp = reinterpret_cast<const float *>(xrow + k4);
                          wp = reinterpret_cast<const float *>(wrows + (clamped_row_offset(row, last) + k4));
@@ -1214,8 +1218,8 @@ static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const f
     // (and the first k of every K range has to be 16-byte aligned)
     p.fast = p.vec_x && p.vec_w && (ldx * fwd::BN < (1ll << 30)) && (ldw * w_rows < (1ll << 30)) &&
              (p.k_per_split % 4 == 0);
-    // (16 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
-    p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 25));
+    // (64 rows of w within 4 GiB: the merge kernel addresses a patch's operands by 32-bit offsets)
+    p.coop = (w_layout == MAM_W_MK) && p.vec_x && p.vec_w && (K % G == 0) && (ldw < (1ll << 24));
     // two groups per recorded span where the resolve is cheap next to the k loop (see mam_fwd_sx_kernel)
     p.gt = (args && use_sx && range_len == 0 && K >= 2048 && K % sx::KT == 0 && p.k_per_split % sx::KT == 0 &&
             option(MAM_OPT_FORWARD_TILING) != MAM_FORWARD_TILING_GROUPS16) ? 2 * G : G;
@@ -1326,7 +1330,9 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
             hipLaunchKernelGGL((mam_fwd_range_sum_kernel<MAM_W_KM, ARGS>), dim3(mb), dim3(256), 0, st, p);
         rc = check_launch("mam_fwd_range_sum_kernel");
     } else if (p.splits > 1) {
-        const unsigned mb = (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
+        // 16 x 16 patches; 4 x 64 with the cooperative resolve
+        const unsigned mb = (ARGS && p.coop) ? (unsigned)(ceil_div(N, 4) * ceil_div(M, 64))
+                                             : (unsigned)(ceil_div(N, 16) * ceil_div(M, 16));
         if (ARGS && p.coop && p.gt == 2 * G)
             hipLaunchKernelGGL((mam_fwd_merge_kernel<MAM_W_MK, ARGS, ARGS, ARGS ? 2 * G : G>), dim3(mb), dim3(256), 0, st, p);
         else if (ARGS && p.coop)
