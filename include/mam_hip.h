@@ -261,6 +261,17 @@ int mam_coo_spmm(const int64_t *row, const int64_t *col, const float *val, int64
                  int64_t ldb, float *c, int64_t R, int64_t K, int64_t C, void *stream);
 
 /*
+ * The sparse operand written out as a dense (R, K) fp32 matrix with row stride ld (cleared first; repeated
+ * coordinates add up).  No counterpart in the reference: from about one stored entry in eight on, the
+ * cusparsemm operator of this build forms a @ b as a dense GEMM of this matrix (the library GEMM of the
+ * platform), which is then faster than any walk over the entries.
+ */
+int mam_csr_to_dense(const int64_t *crow, const int64_t *col, const float *val, float *dense, int64_t ld,
+                     int64_t R, int64_t K, void *stream);
+int mam_coo_to_dense(const int64_t *row, const int64_t *col, const float *val, int64_t nnz, float *dense,
+                     int64_t ld, int64_t R, int64_t K, void *stream);
+
+/*
  * out (N, M) = (alpha * mam_out + beta * mac_out) + bias, each an (N, M) contiguous fp32 array (out may
  * alias mam_out or mac_out), bias (M) or NULL: the vanishing-contribution blend of the module
  * (mamtorch/nn/v4/fullyconnected.py:190-198) in one pass, in the reference's rounding order (two

@@ -34,7 +34,7 @@ EXPORTS = (
     "mam_fc_backward", "mam_selection_count",
     "mam_fc_forward_ranges_workspace", "mam_fc_forward_ranges", "mam_fc_backward_ranges",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward", "mam_csr_validate",
-    "mam_csr_spmm", "mam_coo_spmm",
+    "mam_csr_spmm", "mam_coo_spmm", "mam_csr_to_dense", "mam_coo_to_dense",
     "mam_blend", "mam_apply_keep", "mam_im2col", "mam_col2im",
     "mam_prune_row_offsets", "mam_prune_fill_csr", "mam_prune_apply",
 )
@@ -91,6 +91,8 @@ def lib():
         l.mam_csr_validate.argtypes = [_ptr, _ptr, _i64, _i64, _i64, _ptr, _ptr]
         l.mam_csr_spmm.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
         l.mam_coo_spmm.argtypes = [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
+        l.mam_csr_to_dense.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _ptr]
+        l.mam_coo_to_dense.argtypes = [_ptr, _ptr, _ptr, _i64, _ptr, _i64, _i64, _i64, _ptr]
         _f = ctypes.c_float
         l.mam_prune_row_offsets.argtypes = [_ptr, _i64, _int, _ptr, _ptr, _i64, _f, _ptr, _i64, _i64, _ptr]
         l.mam_prune_fill_csr.argtypes = [_ptr, _i64, _int, _ptr, _ptr, _i64, _f, _ptr, _ptr, _ptr, _i64, _i64, _ptr]
@@ -293,6 +295,23 @@ def coo_spmm(row, col, val, b, R):
     with torch.cuda.device(b.device):
         _check(l.mam_coo_spmm(_p(row), _p(col), _p(val), val.numel(), _p(b), _ld(b), _p(c), R, K, C, _stream(b)))
     return c
+
+
+def csr_to_dense(crow, col, val, R, K):
+    """(R, K) dense fp32 matrix of a CSR operand (repeated coordinates add up)."""
+    l = lib()
+    dense = torch.empty((R, K), dtype=torch.float32, device=val.device)
+    with torch.cuda.device(val.device):
+        _check(l.mam_csr_to_dense(_p(crow), _p(col), _p(val), _p(dense), K, R, K, _stream(val)))
+    return dense
+
+
+def coo_to_dense(row, col, val, R, K):
+    l = lib()
+    dense = torch.empty((R, K), dtype=torch.float32, device=val.device)
+    with torch.cuda.device(val.device):
+        _check(l.mam_coo_to_dense(_p(row), _p(col), _p(val), val.numel(), _p(dense), K, R, K, _stream(val)))
+    return dense
 
 
 def _prune_operands(w, mode, aux, aux2):

@@ -182,6 +182,50 @@ static int check_common(const float *b, int64_t ldb, float *c, int64_t R, int64_
     return MAM_OK;
 }
 
+// Scatter of a sparse matrix into a cleared dense one (repeated coordinates add up).  CSR: a wave per row.
+__global__ __launch_bounds__(NT) void csr_to_dense_kernel(const int64_t *__restrict__ crow, const int64_t *__restrict__ col,
+                                                          const float *__restrict__ val, float *__restrict__ dense,
+                                                          int64_t ld, int R)
+{
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
+    if (r >= R) return;
+    const int64_t beg = crow[r], end = crow[r + 1];
+    float *row = dense + (int64_t)r * ld;
+    for (int64_t e = beg + lane; e < end; e += 64)
+        __hip_atomic_fetch_add(row + col[e], val[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ __launch_bounds__(256) void coo_to_dense_kernel(const int64_t *__restrict__ row, const int64_t *__restrict__ col,
+                                                           const float *__restrict__ val, int64_t nnz,
+                                                           float *__restrict__ dense, int64_t ld)
+{
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < nnz; e += stride)
+        __hip_atomic_fetch_add(dense + row[e] * ld + col[e], val[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+static int check_dense(const float *dense, int64_t ld, int64_t R, int64_t K)
+{
+    if (R < 0 || K < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
+    if (R > INT32_MAX / 2 || K > INT32_MAX / 2) return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
+    if (R == 0 || K == 0) return MAM_OK;
+    if (!dense) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    if (ld < K) return fail(MAM_ERR_INVALID_ARGUMENT, "ld smaller than the number of columns");
+    return MAM_OK;
+}
+
+// rows of `dense` may be strided: cleared row by row when they are
+static int clear_dense(float *dense, int64_t ld, int64_t R, int64_t K, hipStream_t st)
+{
+    if (ld == K) return fill_zero(dense, R * K, st);
+    for (int64_t r = 0; r < R; ++r) {
+        const int rc = fill_zero(dense + r * ld, K, st);
+        if (rc != MAM_OK) return rc;
+    }
+    return MAM_OK;
+}
+
 static bool wide(const float *b, int64_t ldb, const float *c, int64_t C)
 {
     return C % 4 == 0 && ldb % 4 == 0 && (uintptr_t)b % 16 == 0 && (uintptr_t)c % 16 == 0;
@@ -239,4 +283,36 @@ extern "C" int mam_coo_spmm(const int64_t *row, const int64_t *col, const float 
                            row, col, val, nnz, b, ldb, c, (int)C);
     }
     return check_launch("coo_spmm_kernel");
+}
+
+extern "C" int mam_csr_to_dense(const int64_t *crow, const int64_t *col, const float *val, float *dense, int64_t ld,
+                                int64_t R, int64_t K, void *stream)
+{
+    using namespace mam;
+    int rc = spmm::check_dense(dense, ld, R, K);
+    if (rc != MAM_OK || R == 0 || K == 0) return rc;
+    if (!crow) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    rc = spmm::clear_dense(dense, ld, R, K, st);
+    if (rc != MAM_OK) return rc;
+    hipLaunchKernelGGL(spmm::csr_to_dense_kernel, dim3((unsigned)ceil_div(R, spmm::NT / 64)), dim3(spmm::NT), 0, st, crow,
+                       col, val, dense, ld, (int)R);
+    return check_launch("csr_to_dense_kernel");
+}
+
+extern "C" int mam_coo_to_dense(const int64_t *row, const int64_t *col, const float *val, int64_t nnz, float *dense,
+                                int64_t ld, int64_t R, int64_t K, void *stream)
+{
+    using namespace mam;
+    if (nnz < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
+    int rc = spmm::check_dense(dense, ld, R, K);
+    if (rc != MAM_OK || R == 0 || K == 0) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    rc = spmm::clear_dense(dense, ld, R, K, st);
+    if (rc != MAM_OK || nnz == 0) return rc;
+    if (!row || !col || !val) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    int64_t blocks = ceil_div(nnz, 256);
+    if (blocks > 64 * kNumCU) blocks = 64 * kNumCU;
+    hipLaunchKernelGGL(spmm::coo_to_dense_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row, col, val, nnz, dense, ld);
+    return check_launch("coo_to_dense_kernel");
 }

@@ -109,3 +109,39 @@ def test_full_size_against_dense_matmul():
     # linearity, a size-independent property: (2A) @ b == 2 (A @ b) bit for bit (scaling by 2 is exact)
     c2 = capi.csr_spmm(csr.crow_indices(), csr.col_indices(), csr.values() * 2, b, n)
     assert torch.equal(c2, c * 2)
+
+
+@pytest.mark.parametrize("rows,k,rate", [(37, 53, 0.5), (200, 310, 0.7), (5, 1, 0.0), (64, 1000, 0.3), (0, 5, 0.5), (300, 7, 0.99)])
+def test_sparse_operand_written_out_dense(rows, k, rate):
+    """mam_csr_to_dense / mam_coo_to_dense: exact (every cell is one stored value, or the sum of a repeated
+    coordinate's values)."""
+    from mamtorch_amd import capi
+
+    a = _random_sparse(rows, k, rate, seed=rows + k)
+    csr = a.to_sparse_csr()
+    d = capi.csr_to_dense(csr.crow_indices().to(DEV), csr.col_indices().to(DEV), csr.values().to(DEV), rows, k)
+    assert torch.equal(d.cpu(), a + 0.0)           # a + 0.0: the cleared cells are +0
+    coo = a.to_sparse_coo().coalesce()
+    idx = coo.indices()
+    # every coordinate twice, halved values, shuffled: repeated coordinates add up
+    perm = torch.randperm(2 * idx.shape[1], generator=torch.Generator().manual_seed(1))
+    row2, col2 = torch.cat([idx[0], idx[0]])[perm], torch.cat([idx[1], idx[1]])[perm]
+    val2 = torch.cat([coo.values() * 0.5, coo.values() * 0.5])[perm]
+    d2 = capi.coo_to_dense(row2.contiguous().to(DEV), col2.contiguous().to(DEV), val2.contiguous().to(DEV), rows, k)
+    assert torch.equal(d2.cpu(), a + 0.0)
+
+
+@pytest.mark.parametrize("layout", [torch.sparse_csr, torch.sparse_coo])
+@pytest.mark.parametrize("n,l,m,rate", [(300, 500, 260, 0.6), (1024, 2048, 512, 0.7), (129, 64, 64, 0.0), (64, 100, 63, 0.5)])
+def test_operator_at_high_density(layout, n, l, m, rate):
+    """From one stored entry in eight on (and 64 columns of b) the operator writes the operand out dense and
+    calls the library GEMM; (64, 100, 63) stays on the sparse kernels.  Same bar as everywhere: the fp64 product
+    within rtol 1e-5 plus the rounding floor of an fp32 sum."""
+    a = _random_sparse(n, l, rate, seed=n + m).to(DEV)
+    b = torch.randn(l, m, generator=torch.Generator().manual_seed(m)).to(DEV)
+    asparse = a.to_sparse(layout=layout)
+    res = torch.ops.mamtorch_kernel_sparsev1.cusparsemm(asparse, b)
+    assert res.shape == (n, m) and res.dtype == torch.float32
+    want = a.double() @ b.double()
+    floor = a.abs().double() @ b.abs().double()
+    assert bool(((res.double() - want).abs() <= 1e-5 * want.abs() + 2.0 ** -22 * floor).all())
