@@ -24,6 +24,10 @@ Other workloads (`--workload`), same JSON layout, used for the tables in the des
                      dense 4096x4096; one op = one multiply-add; torch.sparse.mm timed beside it
   prune_csr          magnitude pruning of a 4096x4096 weight to 10 % and its compaction to CSR (row offsets +
                      fill); one op = one weight examined; Tensor.to_sparse_csr of the masked weight timed beside it
+  reference_script   the shape and the operator calls of the reference's own timing loop (test/test.py:186-323):
+                     a (128, 2048) x b (2048, 4096) in the reference's (in, out) layout through torch.ops:
+                     v1 fullyconnected, v4 fullyconnected, v4 fullyconnected_fast, v4 fullyconnected_backward with
+                     random indices, torch.matmul beside them; a step = the four MAM operator calls
 """
 import argparse
 import ctypes
@@ -54,7 +58,8 @@ RAMP_MIN_SECONDS = 0.3
 RAMP_MAX_SECONDS = 3.0
 
 WORKLOADS = ("headline", "config1", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
-             "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01", "prune_csr")
+             "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01", "prune_csr",
+             "reference_script")
 
 
 class Layer:
@@ -509,6 +514,50 @@ def run_prune(torch, capi, lib, dev, args):
     return M * K, ms_step, out, cpu
 
 
+def run_reference_script(torch, capi, lib, dev, args):
+    """reference_script: what the reference's test script times (test/test.py:186-323), through the operators of
+    the reference's names and signatures, b in the (in, out) layout.  Each call is timed between events on the
+    stream and, as the script does it, by the host clock around the call and a device synchronize."""
+    N, M, K = 128, 4096, 2048
+    gen = torch.Generator().manual_seed(0)
+    a = torch.randn(N, K, generator=gen).to(dev)
+    b = torch.randn(K, M, generator=gen).to(dev)
+    c = torch.randn(N, M, generator=gen).to(dev)
+    amax = torch.randint(0, K - 1, (N, M), generator=gen, dtype=torch.int32).to(dev)
+    amin = torch.randint(0, K - 1, (N, M), generator=gen, dtype=torch.int32).to(dev)
+    v1, v4 = torch.ops.mamtorch_kernel_v1, torch.ops.mamtorch_kernel_v4
+    phases = [("v1.fullyconnected", lambda: v1.fullyconnected(a, b)),
+              ("v4.fullyconnected", lambda: v4.fullyconnected(a, b)),
+              ("v4.fullyconnected_fast", lambda: v4.fullyconnected_fast(a, b)),
+              ("v4.fullyconnected_backward", lambda: v4.fullyconnected_backward(a, b, c, amax, amin))]
+    stream = torch.cuda.current_stream(dev)
+    ms_step, ph = time_phases(torch, stream, phases, args.steps, args.warmup)
+    _, ph_lib = time_phases(torch, stream, [("torch.matmul", lambda: torch.matmul(a, b))], args.steps, args.warmup)
+    wall = {}
+    for label, fn in phases + [("torch.matmul", lambda: torch.matmul(a, b))]:
+        total = 0.0
+        for _ in range(args.steps):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            total += time.perf_counter() - t0
+        wall[label] = round(total * 1e3 / args.steps, 5)
+    triples = N * K * M
+    out = {
+        "config": {"workload": "the reference's own timing loop: a (128, 2048) ~N(0,1) x b (2048, 4096) ~N(0,1), "
+                               "(in, out) operand as the reference's operators take it; v1 and v4 forward with "
+                               "indices, v4 values-only forward, v4 backward with random indices; one op = one "
+                               "multiply-max-min triple of ONE forward (value = triples / time of the four calls)",
+                   "name": args.workload, "N": N, "K": K, "M": M, "launch": "torch.ops calls"},
+        "phases_ms": {k: round(v, 5) for k, v in ph.items()},
+        "host_clock_ms_per_call_with_synchronize": wall,
+        "library_ms": {k: round(v, 5) for k, v in ph_lib.items()},
+        "roofline": valu_roofline("mamtorch_kernel_v1::fullyconnected (transpose of b + tiling A + merge)", triples,
+                                  ph["v1.fullyconnected"]),
+    }
+    return triples, ms_step, out, None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -524,7 +573,8 @@ def main():
         print("bench.py measures one GPU: the MAM hot path has no multi-GPU part in this build "
               "(--gpus %d refused)" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    small = args.workload in ("headline", "config1", "values_headline", "prune_csr") or args.workload.startswith("sparse")
+    small = args.workload in ("headline", "config1", "values_headline", "prune_csr", "reference_script") \
+        or args.workload.startswith("sparse")
     if args.workload.startswith("spmm"):
         args.steps = 50 if args.steps is None else args.steps
         args.warmup = 20 if args.warmup is None else args.warmup
@@ -546,7 +596,8 @@ def main():
     dev = torch.device("cuda:0")
     lib = capi.lib()
     run = run_sparse if args.workload.startswith("sparse") else run_spmm if args.workload.startswith("spmm") \
-        else run_prune if args.workload == "prune_csr" else run_dense
+        else run_prune if args.workload == "prune_csr" \
+        else run_reference_script if args.workload == "reference_script" else run_dense
     triples, ms_step, extra, cpu = run(torch, capi, lib, dev, args)
 
     out = {
