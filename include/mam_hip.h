@@ -48,12 +48,15 @@ extern "C" {
                                  likewise for min (the retired convolution modules' literal rule)        */
 
 /* Run-time switches for mam_set_option().  Their initial values come from the environment variables of
- * the same names (MAM_FORWARD_TILING = auto | wide | 2, MAM_BACKWARD_FORK = 0 | 1, MAM_BACKWARD_ONE_LAUNCH = 0 | 1), read once when the
- * library is loaded. */
+ * the same names, read once when the library is loaded: MAM_FORWARD_TILING = auto | wide | 0 | 1 | 2,
+ * MAM_BACKWARD_FORK = auto | -1 | 0 | 1, MAM_BACKWARD_ONE_LAUNCH = auto | 0 (off) | 1 (auto) | 2 (on),
+ * MAM_BACKWARD_EXACT = 0 | 1.  A value outside an
+ * option's range is refused by mam_set_option() and ignored (with the default kept) in the environment. */
 #define MAM_OPT_FORWARD_TILING 0 /* which dense forward tiling serves a call                      */
 #define MAM_OPT_BACKWARD_FORK 1  /* x_grad on the library's second stream beside w_grad           */
 #define MAM_OPT_BACKWARD_ONE_LAUNCH 2 /* both gradients in one launch where the shape allows it    */
-#define MAM_OPT_COUNT_ 3
+#define MAM_OPT_BACKWARD_EXACT 3 /* w_grad accumulated in 64-bit fixed-point cells (exact sums)    */
+#define MAM_OPT_COUNT_ 4
 #define MAM_FORWARD_TILING_AUTO 0 /* wave-uniform-rows tiling where the layout allows it           */
 #define MAM_FORWARD_TILING_WIDE 1 /* every call on the general 64 x 128 tiling                     */
 #define MAM_FORWARD_TILING_GROUPS16 2 /* as AUTO, but indices recorded per 16 products at every K   */
@@ -64,6 +67,9 @@ extern "C" {
 #define MAM_BACKWARD_ONE_LAUNCH_AUTO 1 /* small calls only (<= 2^16 outputs), where the launches are the cost */
 #define MAM_BACKWARD_ONE_LAUNCH_ON 2   /* wherever the shape allows it: (M,K) weights, 16-byte aligned operands,
                                           batch below 2 x CUs, K <= 4096 */
+#define MAM_BACKWARD_EXACT_OFF 0 /* w_grad in fp32 cells: each sum within the rounding floor of its order    */
+#define MAM_BACKWARD_EXACT_ON 1  /* w_grad = the exact sum of its fp32 terms rounded once (about twice the
+                                    kernel time at 256 x 4096 x 4096); (M,K) weights with hand-over only     */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int mam_version(void);

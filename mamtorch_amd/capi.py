@@ -18,6 +18,7 @@ PRUNE_COUNT = 2
 OPT_FORWARD_TILING = 0
 OPT_BACKWARD_FORK = 1
 OPT_BACKWARD_ONE_LAUNCH = 2
+OPT_BACKWARD_EXACT = 3
 FORWARD_TILING_AUTO = 0
 FORWARD_TILING_WIDE = 1
 FORWARD_TILING_GROUPS16 = 2

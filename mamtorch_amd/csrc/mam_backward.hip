@@ -623,7 +623,7 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
 {
     int rc = MAM_OK;
     if (planes <= 1) range_len = (int)K;
-    const int dev = ensure_device();
+    const int dev = ensure_device(st);
     if (dev < 0) return dev;
     const int lds_cap = g_lds_floats[dev];
     const int cus = num_cus();
@@ -722,7 +722,7 @@ static int launch_both(const float *x, int64_t ldx, const float *w, int64_t ldw,
                        int range_len, bool auto_mode)
 {
     if (planes <= 1) range_len = (int)K;
-    const int dev = ensure_device();
+    const int dev = ensure_device(st);
     if (dev < 0) return dev;
     const int cus = num_cus();
     const bool vec_in = (M % 4 == 0) && (N * M % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
@@ -761,7 +761,7 @@ static int launch_both(const float *x, int64_t ldx, const float *w, int64_t ldw,
 int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t *argmin, const float *w_sel,
                          float *x_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
 {
-    const int dev = ensure_device();
+    const int dev = ensure_device(st);
     if (dev < 0) return dev;
     const int cells_cap = (g_lds_floats[dev] - 2048) / 2;
     const int kc = (int)(K < cells_cap ? K : cells_cap);

@@ -27,7 +27,9 @@ constexpr int kMaxDevices = 16;
 typedef int (*DeviceHook)(int dev);
 struct DeviceHookRegistration { explicit DeviceHookRegistration(DeviceHook fn); };
 // Returns the current device's index (0..kMaxDevices-1) after its hooks have run, or a negative MAM_ERR_*.
-int ensure_device();
+// `st` is the stream the entry point launches on: while it is being captured the hooks still run (they
+// create nothing), and the second stream and its events are left for the first call outside a capture.
+int ensure_device(hipStream_t st = nullptr);
 
 // Run-time switches (mam_set_option; initial values come from the environment, read once at load).
 int option(int which);

@@ -104,12 +104,12 @@ int transpose(const float *src, int64_t ld, float *dst, int64_t rows, int64_t co
 namespace {
 struct DeviceState {
     std::mutex lock;             // set-up of this device, and its fork/join sequences
-    std::atomic<int> ready{0};   // 1 once every hook has run
+    std::atomic<int> ready{0};   // 1 once every hook has run, 2 once the second stream exists as well
     int rc = MAM_OK;
     std::atomic<int> cus{0};     // compute units, 0 = not asked yet
     hipStream_t stream = nullptr;   // the library's second stream (default priority)
     hipEvent_t fork = nullptr, join = nullptr;
-    bool side_ok = false;
+    bool side_ok = false, side_tried = false;
 };
 DeviceState g_devices[kMaxDevices];
 
@@ -117,19 +117,32 @@ constexpr int kMaxHooks = 16;
 DeviceHook g_hooks[kMaxHooks];
 int g_num_hooks = 0;
 
-int env_choice(const char *name, int fallback)
+// The values each option accepts.
+struct OptionRange { const char *env; int lo, hi, fallback; bool wide_word; };
+constexpr OptionRange kOptionRanges[MAM_OPT_COUNT_] = {
+    {"MAM_FORWARD_TILING", MAM_FORWARD_TILING_AUTO, MAM_FORWARD_TILING_GROUPS16, MAM_FORWARD_TILING_AUTO, true},
+    {"MAM_BACKWARD_FORK", MAM_BACKWARD_FORK_AUTO, MAM_BACKWARD_FORK_ON, MAM_BACKWARD_FORK_AUTO, false},
+    {"MAM_BACKWARD_ONE_LAUNCH", MAM_BACKWARD_ONE_LAUNCH_OFF, MAM_BACKWARD_ONE_LAUNCH_ON, MAM_BACKWARD_ONE_LAUNCH_AUTO,
+     false},
+    {"MAM_BACKWARD_EXACT", MAM_BACKWARD_EXACT_OFF, MAM_BACKWARD_EXACT_ON, MAM_BACKWARD_EXACT_OFF, false},
+};
+
+// An option's initial value: its environment variable when that holds "auto", a number inside the option's
+// range or (forward tiling only) "wide"; the default otherwise.
+int env_choice(int which)
 {
-    const char *v = getenv(name);
-    if (!v || !v[0]) return fallback;
-    if (strcmp(v, "wide") == 0) return MAM_FORWARD_TILING_WIDE;
-    if (strcmp(v, "auto") == 0) return fallback;
-    return atoi(v);
+    const OptionRange &r = kOptionRanges[which];
+    const char *v = getenv(r.env);
+    if (!v || !v[0] || strcmp(v, "auto") == 0) return r.fallback;
+    if (r.wide_word && strcmp(v, "wide") == 0) return MAM_FORWARD_TILING_WIDE;
+    char *end = nullptr;
+    const long n = strtol(v, &end, 10);
+    if (end == v || *end != '\0' || n < r.lo || n > r.hi) return r.fallback;
+    return (int)n;
 }
 // initial values from the environment, read once when the library is loaded
 std::atomic<int> g_options[MAM_OPT_COUNT_] = {
-    {env_choice("MAM_FORWARD_TILING", MAM_FORWARD_TILING_AUTO)},
-    {env_choice("MAM_BACKWARD_FORK", MAM_BACKWARD_FORK_AUTO)},
-    {env_choice("MAM_BACKWARD_ONE_LAUNCH", MAM_BACKWARD_ONE_LAUNCH_AUTO)},
+    {env_choice(0)}, {env_choice(1)}, {env_choice(2)}, {env_choice(3)},
 };
 }  // namespace
 
@@ -140,7 +153,27 @@ DeviceHookRegistration::DeviceHookRegistration(DeviceHook fn)
 
 int option(int which) { return g_options[which].load(std::memory_order_relaxed); }
 
-int ensure_device()
+// Whether `st`, the stream an entry point launches on, is being captured into a graph.
+static bool stream_is_capturing(hipStream_t st)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return status == hipStreamCaptureStatusActive;
+}
+
+static void create_side_stream(DeviceState &d)
+{
+    d.side_ok = hipStreamCreateWithFlags(&d.stream, hipStreamNonBlocking) == hipSuccess &&
+                hipEventCreateWithFlags(&d.fork, hipEventDisableTiming) == hipSuccess &&
+                hipEventCreateWithFlags(&d.join, hipEventDisableTiming) == hipSuccess;
+    if (!d.side_ok) (void)hipGetLastError();
+    d.side_tried = true;
+}
+
+int ensure_device(hipStream_t st)
 {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) {
@@ -149,16 +182,22 @@ int ensure_device()
     }
     if (dev < 0 || dev >= kMaxDevices) return fail(MAM_ERR_UNSUPPORTED, "device index %d beyond %d", dev, kMaxDevices - 1);
     DeviceState &d = g_devices[dev];
-    if (d.ready.load(std::memory_order_acquire)) return d.rc == MAM_OK ? dev : d.rc;
+    if (d.ready.load(std::memory_order_acquire) == 2) return d.rc == MAM_OK ? dev : d.rc;
+    // The kernel attributes and the scratch array's address may be taken at any time; the second stream and
+    // its events must not be created while the caller's stream is being captured: that part waits for the
+    // first call outside a capture (until then nothing forks).
+    const bool capturing = stream_is_capturing(st);
     std::lock_guard<std::mutex> hold(d.lock);
-    if (!d.ready.load(std::memory_order_relaxed)) {
-        d.side_ok = hipStreamCreateWithFlags(&d.stream, hipStreamNonBlocking) == hipSuccess &&
-                    hipEventCreateWithFlags(&d.fork, hipEventDisableTiming) == hipSuccess &&
-                    hipEventCreateWithFlags(&d.join, hipEventDisableTiming) == hipSuccess;
-        if (!d.side_ok) (void)hipGetLastError();
+    int state = d.ready.load(std::memory_order_relaxed);
+    if (state == 0) {
         for (int i = 0; i < g_num_hooks && d.rc == MAM_OK; ++i) d.rc = g_hooks[i](dev);
-        d.ready.store(1, std::memory_order_release);
+        state = 1;
     }
+    if (state == 1 && !capturing) {
+        create_side_stream(d);
+        state = 2;
+    }
+    d.ready.store(state, std::memory_order_release);
     return d.rc == MAM_OK ? dev : d.rc;
 }
 
@@ -194,7 +233,7 @@ ForkedStream::ForkedStream(hipStream_t st, int64_t units)
         want = units >= (1 << 22) || (capturing == hipStreamCaptureStatusActive && units >= (1 << 16));
     }
     if (!want) return;
-    const int dev = ensure_device();
+    const int dev = ensure_device(st);
     if (dev < 0 || !g_devices[dev].side_ok) return;
     DeviceState &d = g_devices[dev];
     d.lock.lock();
@@ -261,6 +300,9 @@ extern "C" int mam_device_info(int *compute_units, int *max_clock_khz)
 extern "C" int mam_set_option(int option, int value)
 {
     if (option < 0 || option >= MAM_OPT_COUNT_) return mam::fail(MAM_ERR_INVALID_ARGUMENT, "unknown option %d", option);
+    const mam::OptionRange &r = mam::kOptionRanges[option];
+    if (value < r.lo || value > r.hi)
+        return mam::fail(MAM_ERR_INVALID_ARGUMENT, "option %d takes values %d..%d, got %d", option, r.lo, r.hi, value);
     mam::g_options[option].store(value, std::memory_order_relaxed);
     return MAM_OK;
 }

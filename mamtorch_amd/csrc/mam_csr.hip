@@ -280,32 +280,77 @@ __global__ __launch_bounds__(NT_F) void csr_fwd_kernel(
         // extreme itself, which equals the second product -- except that a zero extreme may carry the
         // other zero's sign, so a second entry selected for a zero extreme is recomputed (rare: a branch
         // that whole waves skip).
+        // All 2 TI outputs of the lane are settled together: their column / value loads leave in one
+        // batch and the selected inputs in a second one, so the epilogue is two trips to memory and not
+        // one chain of dependent loads per output.
         int ri[2][TI];
         float rw[2][TI], rx[2][TI];
+        if (nnz > 0) {
+            int es[2][TI];
+            bool ok[2][TI], first[2][TI];
 #pragma unroll
-        for (int t = 0; t < TI; ++t) {
+            for (int t = 0; t < TI; ++t) {
 #pragma unroll
-            for (int ext = 0; ext < 2; ++ext) {
-                const int pair = ext ? pmin[t] : pmax[t];
-                const float kept = ext ? amin[t] : amax[t];
-                float &target = ext ? vmin[t] : vmax[t];
-                int &pos = ext ? pmin[t] : pmax[t];
-                if (nnz > 0 && pair >= 0) {
-                    const bool first = kept == target;
-                    const int e0 = 2 * pair, e = first ? e0 : ((e0 + 1 < nnz) ? e0 + 1 : e0);
-                    const int64_t cc = col[beg + e];
-                    const float w = val[beg + e];
-                    if (first) {
-                        target = kept;
-                    } else if (target == 0.0f) {
-                        target = xT[cc * (int64_t)ldt + nl + t] * w;
+                for (int ext = 0; ext < 2; ++ext) {
+                    const int pair = ext ? pmin[t] : pmax[t];
+                    const float kept = ext ? amin[t] : amax[t], target = ext ? vmin[t] : vmax[t];
+                    ok[ext][t] = pair >= 0;
+                    first[ext][t] = kept == target;
+                    const int e0 = 2 * (pair < 0 ? 0 : pair);
+                    es[ext][t] = first[ext][t] ? e0 : ((e0 + 1 < nnz) ? e0 + 1 : e0);
+                }
+            }
+            int64_t cc[2][TI];
+#pragma unroll
+            for (int t = 0; t < TI; ++t) {
+#pragma unroll
+                for (int ext = 0; ext < 2; ++ext) {
+                    cc[ext][t] = col[beg + es[ext][t]];
+                    rw[ext][t] = val[beg + es[ext][t]];
+                }
+            }
+            bool need_x = x_sel != nullptr;
+            if (!need_x) {
+                // a second entry selected for a zero extreme is recomputed (rare: whole waves skip the loads)
+                bool rare = false;
+#pragma unroll
+                for (int t = 0; t < TI; ++t) {
+                    rare = rare || (ok[0][t] && !first[0][t] && vmax[t] == 0.0f);
+                    rare = rare || (ok[1][t] && !first[1][t] && vmin[t] == 0.0f);
+                }
+                need_x = __ballot(rare) != 0ull;
+            }
+#pragma unroll
+            for (int t = 0; t < TI; ++t) {
+#pragma unroll
+                for (int ext = 0; ext < 2; ++ext) rx[ext][t] = need_x ? xT[cc[ext][t] * (int64_t)ldt + nl + t] : 0.0f;
+            }
+#pragma unroll
+            for (int t = 0; t < TI; ++t) {
+#pragma unroll
+                for (int ext = 0; ext < 2; ++ext) {
+                    float &target = ext ? vmin[t] : vmax[t];
+                    int &pos = ext ? pmin[t] : pmax[t];
+                    if (ok[ext][t]) {
+                        if (first[ext][t]) target = ext ? amin[t] : amax[t];
+                        else if (target == 0.0f) target = rx[ext][t] * rw[ext][t];
+                        pos = es[ext][t];
+                        ri[ext][t] = (int)cc[ext][t];
+                        if (!x_sel) rx[ext][t] = 0.0f;
+                    } else {
+                        pos = -1;
+                        ri[ext][t] = -1;
+                        rw[ext][t] = 0.0f;
+                        rx[ext][t] = 0.0f;
                     }
-                    pos = e;
-                    ri[ext][t] = (int)cc;
-                    rw[ext][t] = w;
-                    rx[ext][t] = x_sel ? xT[cc * (int64_t)ldt + nl + t] : 0.0f;
-                } else {
-                    pos = -1;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < TI; ++t) {
+#pragma unroll
+                for (int ext = 0; ext < 2; ++ext) {
+                    (ext ? pmin[t] : pmax[t]) = -1;
                     ri[ext][t] = -1;
                     rw[ext][t] = 0.0f;
                     rx[ext][t] = 0.0f;
@@ -766,7 +811,7 @@ extern "C" int mam_csr_fc_forward(const float *x, int64_t ldx, const int64_t *cr
     if (!workspace || workspace_bytes < need || (uintptr_t)workspace % 16 != 0)
         return fail(MAM_ERR_WORKSPACE, "CSR forward needs %zu workspace bytes, 16-byte aligned, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
-    const int dev = ensure_device();
+    const int dev = ensure_device(static_cast<hipStream_t>(stream));
     if (dev < 0) return dev;
     hipStream_t st = static_cast<hipStream_t>(stream);
     float *xT = static_cast<float *>(workspace);
@@ -841,7 +886,7 @@ extern "C" int mam_csr_fc_backward(const float *x, int64_t ldx, const int64_t *c
         const int rc_join = fork.join();
         return rc != MAM_OK ? rc : rc_join;
     }
-    const int dev = ensure_device();
+    const int dev = ensure_device(st);
     if (dev < 0) return dev;
     const int budget = csr::g_bwd_lds_floats[dev];
     const int kc = (int)(K < budget ? K : budget);

@@ -72,11 +72,20 @@ struct Params {
     int gt;            // products per recorded group: G, or 2 G on the wave-uniform-rows tiling at large K
 };
 
+// An extreme that still holds its initial value (-inf for the max, +inf for the min) was never strictly
+// improved: every product was NaN or equal to that infinity.  The ordered compares of a scalar scan
+// (mamtorch/kernel/v1/csrc/cuda/fullyconnected.cu:132-142) leave the index at the first k of the range in
+// that case, and so does the resolve: it looks for no match then.
+__device__ __forceinline__ bool never_improved(float target, bool is_min)
+{
+    return target == (is_min ? __builtin_inff() : -__builtin_inff());
+}
+
 // First k in group g (ascending) whose product equals `target`; value recomputed from it.
 // The cost of this step is the number of cache lines each wave touches, not arithmetic, so the
 // G operands of each side are fetched with 16-byte loads when the layout allows it.
 template <int LAYOUT>
-__device__ __forceinline__ void resolve(const Params &p, int n, int m, int kb, int klast, float target,
+__device__ __forceinline__ void resolve(const Params &p, int n, int m, int kb, int klast, float target, bool is_min,
                                         float &val, int &idx, float &wsel, float &xsel)
 {
     // the group is k = kb .. kb + G - 1; k beyond klast (the last k of the scanned range) repeat klast
@@ -109,10 +118,11 @@ __device__ __forceinline__ void resolve(const Params &p, int n, int m, int kb, i
         for (int kk = 0; kk < G; ++kk)
             wv[kk] = load_w<LAYOUT>(p.w, p.ldw, (kb + kk) < klast ? (kb + kk) : klast, m);
     }
+    const bool never = never_improved(target, is_min);
 #pragma unroll
     for (int kk = G - 1; kk >= 0; --kk) {
         const float prod = xv[kk] * wv[kk];
-        if (prod == target) { idx = (kb + kk) < klast ? (kb + kk) : klast; val = prod; wsel = wv[kk]; xsel = xv[kk]; }
+        if (prod == target && !never) { idx = (kb + kk) < klast ? (kb + kk) : klast; val = prod; wsel = wv[kk]; xsel = xv[kk]; }
     }
 }
 
@@ -140,8 +150,8 @@ __device__ __forceinline__ void finish(const Params &p, int n, int m, float vmax
     int ih = 0, il = 0;
     float wh = 0.0f, wl = 0.0f, xh = 0.0f, xl = 0.0f;
     if (ARGS) {
-        resolve<LAYOUT>(p, n, m, gmax * G, p.K - 1, vmax, hi, ih, wh, xh);
-        resolve<LAYOUT>(p, n, m, gmin * G, p.K - 1, vmin, lo, il, wl, xl);
+        resolve<LAYOUT>(p, n, m, gmax * G, p.K - 1, vmax, false, hi, ih, wh, xh);
+        resolve<LAYOUT>(p, n, m, gmin * G, p.K - 1, vmin, true, lo, il, wl, xl);
     } else {
         if (hi == 0.0f) hi = first_zero_product<LAYOUT>(p.x + (int64_t)n * p.ldx, p.w, p.ldw, m, 0, p.K);
         if (lo == 0.0f) lo = first_zero_product<LAYOUT>(p.x + (int64_t)n * p.ldx, p.w, p.ldw, m, 0, p.K);
@@ -247,8 +257,10 @@ __device__ __forceinline__ void resolve_wave(const Params &p, const float *vals,
                 if (p1 == target[b]) { key = k0 + 1; wsel = wa[b][v].y; xsel = xa[b][v].y; }
                 if (p0 == target[b]) { key = k0 + 0; wsel = wa[b][v].x; xsel = xa[b][v].x; }
             }
+            if (never_improved(target[b], ext != 0)) key = 255;
             const int best = quad_min(key);
-            // no product equals the extreme (NaN operands): the first k of the group, from lane 0
+            // no product equals the extreme (NaN operands), or the extreme was never improved: the first k of
+            // the group, from lane 0
             const bool fallback = best == 255 && sub == 0;
             if ((key == best && key != 255) || fallback) {
                 // the value is recomputed from the selected operands (the sign of a zero follows them)
@@ -782,8 +794,8 @@ __global__ __launch_bounds__(256) void mam_fwd_range_sum_kernel(const Params p)
             const int pk = __float_as_int(base[2 * nm + o]);
             int ih, il;
             float w_unused, x_unused;
-            resolve<LAYOUT>(p, n, m, kb + (pk & 0xffff) * G, ke - 1, hi, hi, ih, w_unused, x_unused);
-            resolve<LAYOUT>(p, n, m, kb + ((pk >> 16) & 0xffff) * G, ke - 1, lo, lo, il, w_unused, x_unused);
+            resolve<LAYOUT>(p, n, m, kb + (pk & 0xffff) * G, ke - 1, hi, false, hi, ih, w_unused, x_unused);
+            resolve<LAYOUT>(p, n, m, kb + ((pk >> 16) & 0xffff) * G, ke - 1, lo, true, lo, il, w_unused, x_unused);
             p.argmax[(int64_t)s * nm + o] = ih;
             p.argmin[(int64_t)s * nm + o] = il;
         } else {
@@ -1296,7 +1308,7 @@ static int launch(const float *x, int64_t ldx, const float *w, int64_t ldw, int 
 
     const int64_t nblk = (int64_t)p.tiles_n * p.tiles_m * p.splits;
     if (nblk > INT32_MAX) return fail(MAM_ERR_UNSUPPORTED, "too many tiles");
-    const int dev = ensure_device();
+    const int dev = ensure_device(static_cast<hipStream_t>(stream));
     if (dev < 0) return dev;
     char *scratch_base = static_cast<char *>(workspace);
     if (static_scratch && wt_bytes + need > 0) {
@@ -1402,19 +1414,10 @@ extern "C" int mam_fc_forward_ranges(const float *x, int64_t ldx, const float *w
                               workspace_bytes, stream, false, range_len);
 }
 
-extern "C" int mam_fc_forward_describe(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
-                                       int64_t N, int64_t K, int64_t M, int with_indices, char *text, size_t text_bytes)
+static void describe_plan(const mam::fwd::Plan &plan, int w_layout, int64_t K, bool with_indices, char *text,
+                          size_t text_bytes)
 {
     using namespace mam;
-    fwd::Plan plan;
-    const int rc = fwd::make_plan(plan, with_indices != 0, x, ldx, w, ldw, w_layout, nullptr, nullptr, nullptr,
-                                  nullptr, nullptr, nullptr, N, K, M);
-    if (rc != MAM_OK) return rc;
-    if (!text || text_bytes == 0) return fail(MAM_ERR_INVALID_ARGUMENT, "no text buffer");
-    if (N == 0 || M == 0) {
-        snprintf(text, text_bytes, "nothing to launch");
-        return MAM_OK;
-    }
     const fwd::Params &p = plan.p;
     const char *what = with_indices ? "args" : "values";
     if (plan.use_sx)
@@ -1430,6 +1433,42 @@ extern "C" int mam_fc_forward_describe(const float *x, int64_t ldx, const float 
                  p.splits, p.k_per_split, (with_indices && p.coop) ? "cooperative resolve" : "per-thread resolve",
                  plan.need);
     }
+}
+
+extern "C" int mam_fc_forward_describe(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                                       int64_t N, int64_t K, int64_t M, int with_indices, char *text, size_t text_bytes)
+{
+    using namespace mam;
+    fwd::Plan plan;
+    const int rc = fwd::make_plan(plan, with_indices != 0, x, ldx, w, ldw, w_layout, nullptr, nullptr, nullptr,
+                                  nullptr, nullptr, nullptr, N, K, M);
+    if (rc != MAM_OK) return rc;
+    if (!text || text_bytes == 0) return fail(MAM_ERR_INVALID_ARGUMENT, "no text buffer");
+    if (N == 0 || M == 0) {
+        snprintf(text, text_bytes, "nothing to launch");
+        return MAM_OK;
+    }
+    // A (K, M) operand is transposed once into the workspace when that has room (what
+    // mam_fc_forward_workspace_for() asks for) and the wave-uniform-rows tiling then runs on the copy: both
+    // routes are named, the one a call takes depends on the workspace it brings.
+    if (w_layout == MAM_W_KM && fwd::transposed_operand_pays(N, K, M)) {
+        fwd::Plan tplan;
+        float *const aligned = reinterpret_cast<float *>((uintptr_t)256);
+        const int trc = fwd::make_plan(tplan, with_indices != 0, x, ldx, aligned, K, MAM_W_MK, nullptr, nullptr,
+                                       nullptr, nullptr, nullptr, nullptr, N, K, M);
+        if (trc == MAM_OK && tplan.use_sx) {
+            const size_t copy = ((size_t)M * (size_t)K * sizeof(float) + 255) / 256 * 256;
+            int used = snprintf(text, text_bytes, "with %zu workspace bytes: transpose_kernel + ", copy + tplan.need);
+            if (used < 0 || (size_t)used >= text_bytes) return MAM_OK;
+            describe_plan(tplan, MAM_W_MK, K, with_indices != 0, text + used, text_bytes - used);
+            used = (int)strlen(text);
+            const int more = snprintf(text + used, text_bytes - used, "; with less: ");
+            if (more < 0 || (size_t)(used + more) >= text_bytes) return MAM_OK;
+            describe_plan(plan, w_layout, K, with_indices != 0, text + used + more, text_bytes - used - more);
+            return MAM_OK;
+        }
+    }
+    describe_plan(plan, w_layout, K, with_indices != 0, text, text_bytes);
     return MAM_OK;
 }
 

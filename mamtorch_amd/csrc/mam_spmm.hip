@@ -183,26 +183,34 @@ static int check_common(const float *b, int64_t ldb, float *c, int64_t R, int64_
 }
 
 // Scatter of a sparse matrix into a cleared dense one (repeated coordinates add up).  CSR: a wave per row.
+// These kernels WRITE at the coordinates they are given, so an entry whose column (or row) lies outside the
+// matrix is skipped: nothing is ever written outside `dense`.
 __global__ __launch_bounds__(NT) void csr_to_dense_kernel(const int64_t *__restrict__ crow, const int64_t *__restrict__ col,
                                                           const float *__restrict__ val, float *__restrict__ dense,
-                                                          int64_t ld, int R)
+                                                          int64_t ld, int R, int K)
 {
     const int lane = threadIdx.x & 63;
     const int r = blockIdx.x * (NT / 64) + (threadIdx.x >> 6);
     if (r >= R) return;
     const int64_t beg = crow[r], end = crow[r + 1];
     float *row = dense + (int64_t)r * ld;
-    for (int64_t e = beg + lane; e < end; e += 64)
-        __hip_atomic_fetch_add(row + col[e], val[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int64_t e = beg + lane; e < end; e += 64) {
+        const int64_t cc = col[e];
+        if ((uint64_t)cc < (uint64_t)K)
+            __hip_atomic_fetch_add(row + cc, val[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 __global__ __launch_bounds__(256) void coo_to_dense_kernel(const int64_t *__restrict__ row, const int64_t *__restrict__ col,
                                                            const float *__restrict__ val, int64_t nnz,
-                                                           float *__restrict__ dense, int64_t ld)
+                                                           float *__restrict__ dense, int64_t ld, int R, int K)
 {
     const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < nnz; e += stride)
-        __hip_atomic_fetch_add(dense + row[e] * ld + col[e], val[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < nnz; e += stride) {
+        const int64_t rr = row[e], cc = col[e];
+        if ((uint64_t)rr < (uint64_t)R && (uint64_t)cc < (uint64_t)K)
+            __hip_atomic_fetch_add(dense + rr * ld + cc, val[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 static int check_dense(const float *dense, int64_t ld, int64_t R, int64_t K)
@@ -296,7 +304,7 @@ extern "C" int mam_csr_to_dense(const int64_t *crow, const int64_t *col, const f
     rc = spmm::clear_dense(dense, ld, R, K, st);
     if (rc != MAM_OK) return rc;
     hipLaunchKernelGGL(spmm::csr_to_dense_kernel, dim3((unsigned)ceil_div(R, spmm::NT / 64)), dim3(spmm::NT), 0, st, crow,
-                       col, val, dense, ld, (int)R);
+                       col, val, dense, ld, (int)R, (int)K);
     return check_launch("csr_to_dense_kernel");
 }
 
@@ -313,6 +321,7 @@ extern "C" int mam_coo_to_dense(const int64_t *row, const int64_t *col, const fl
     if (!row || !col || !val) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
     int64_t blocks = ceil_div(nnz, 256);
     if (blocks > 64 * kNumCU) blocks = 64 * kNumCU;
-    hipLaunchKernelGGL(spmm::coo_to_dense_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row, col, val, nnz, dense, ld);
+    hipLaunchKernelGGL(spmm::coo_to_dense_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row, col, val, nnz, dense, ld,
+                       (int)R, (int)K);
     return check_launch("coo_to_dense_kernel");
 }

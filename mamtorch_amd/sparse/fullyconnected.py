@@ -64,7 +64,9 @@ def validate_csr(w_csr: Tensor) -> None:
     a row.  The operators themselves do not check (a check needs a device round trip per call, and
     ``torch.sparse_csr_tensor`` builds unchecked tensors by default), so call this once on a tensor that
     did not come from ``Tensor.to_sparse_csr()`` / ``sparse.prune`` before handing it to them: a malformed
-    tensor makes the kernels read, and the COO SpMM write, out of range."""
+    tensor makes the kernels read out of range, and the COO SpMM write out of range (its result rows come
+    from the row indices).  The dense route of ``cusparsemm`` (``mam_csr_to_dense`` / ``mam_coo_to_dense``)
+    writes too, and for that reason drops every entry whose coordinates lie outside the matrix."""
     from .. import capi
 
     if w_csr.layout != torch.sparse_csr or w_csr.dim() != 2:

@@ -22,12 +22,20 @@ def forward(x, b, bias=None):
     for n in range(N):
         for m in range(M):
             prods = [f32(x[n, k]) * f32(b[k, m]) for k in range(K)]
-            hi, lo, ih, il = prods[0], prods[0], 0, 0
-            for k in range(1, K):
-                if prods[k] > hi:
-                    hi, ih = prods[k], k
-                if prods[k] < lo:
-                    lo, il = prods[k], k
+            # NaN products take no part (the reference kernel compares with ordered > and <).  Among the
+            # rest the extreme is the largest / smallest value and its index the lowest k that holds it;
+            # an extreme that does not rise above -inf (fall below +inf) -- no candidates at all, or only
+            # that infinity -- keeps the scan's starting index 0.
+            real = [(k, p) for k, p in enumerate(prods) if p == p]
+            hi = max([p for _, p in real], default=f32(-np.inf))
+            lo = min([p for _, p in real], default=f32(np.inf))
+            ih = min([k for k, p in real if p == hi], default=0) if hi > -np.inf else 0
+            il = min([k for k, p in real if p == lo], default=0) if lo < np.inf else 0
+            # a zero extreme carries the sign of the FIRST zero product
+            if hi == 0:
+                hi = prods[ih]
+            if lo == 0:
+                lo = prods[il]
             s = f32(hi + lo)
             if bias is not None:
                 s = f32(s + f32(bias[m]))

@@ -48,7 +48,15 @@ static inline float w_at(const float *w, int64_t ldw, int layout, int64_t k, int
     return layout == MAM_W_MK ? w[m * ldw + k] : w[k * ldw + m];
 }
 
-/* y[n,m] = (max_k x[n,k]*w[k,m] + min_k x[n,k]*w[k,m]) + bias[m]; first-index ties. */
+/*
+ * y[n,m] = (max_k x[n,k]*w[k,m] + min_k x[n,k]*w[k,m]) + bias[m]; first-index ties.
+ * The scan is the reference kernel's (mamtorch/kernel/v1/csrc/cuda/fullyconnected.cu:68-78,132-142): the
+ * accumulators start below / above every float with index 0 (the reference starts the max at FLT_MIN, a bug
+ * that the build does not reproduce: -inf here), k ascends, and a product replaces an extreme only when an
+ * ORDERED compare says it is strictly greater / smaller.  A NaN product therefore never wins and never
+ * sticks, wherever it stands; a column of NaN products keeps (-inf, index 0) and (+inf, index 0), and so
+ * does an extreme whose only candidates equal the starting infinity.
+ */
 void mam_oracle_forward(const float *x, int64_t ldx, const float *w, int64_t ldw, int layout,
                         const float *bias, float *c, int32_t *argmax, int32_t *argmin,
                         int64_t N, int64_t K, int64_t M)
@@ -56,11 +64,10 @@ void mam_oracle_forward(const float *x, int64_t ldx, const float *w, int64_t ldw
 #pragma omp parallel for schedule(static)
     for (int64_t n = 0; n < N; ++n) {
         for (int64_t m = 0; m < M; ++m) {
-            float vmax = 0.f, vmin = 0.f;
+            float vmax = -__builtin_inff(), vmin = __builtin_inff();
             int32_t imax = 0, imin = 0;
             for (int64_t k = 0; k < K; ++k) {
                 volatile float p = x[n * ldx + k] * w_at(w, ldw, layout, k, m);
-                if (k == 0) { vmax = p; vmin = p; continue; }
                 if (p > vmax) { vmax = p; imax = (int32_t)k; }
                 if (p < vmin) { vmin = p; imin = (int32_t)k; }
             }

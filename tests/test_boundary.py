@@ -6,6 +6,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -128,9 +129,11 @@ def test_fake_kernels_propagate_shapes():
 
 
 def test_module_constructor_and_repr():
+    torch.manual_seed(0)
     layer = mt.nn.FullyConnected(784, 256)
     assert layer.weight.shape == (256, 784) and layer.bias.shape == (256,)
-    bound = 1 / 784 ** 0.5
+    # the draws are fp32: the largest one can round up to the fp32 value of the bound
+    bound = float(np.float32(1 / 784 ** 0.5))
     assert float(layer.weight.detach().abs().max()) <= bound and float(layer.bias.detach().abs().max()) <= bound
     assert (layer.beta, layer.alpha) == (0.0, 1.0)
     assert repr(layer) == "MAM@FullyConnected(in_features=784, out_features=256, bias=True)"
@@ -206,7 +209,8 @@ def test_legacy_layers_constructors_schedules_and_names():
     for want in (0.75, 0.5, 0.25, 0):
         layer.vcon_step()
         assert layer.beta == want
-    bound = (6 / (2 + 6)) ** 0.5
+    bound = float(np.float32((6 / (2 + 6)) ** 0.5))
+    torch.manual_seed(0)
     uniform = mt.nn.v1.FullyConnected(50, 6)
     assert float(uniform.weight.abs().max()) <= bound and uniform.beta == 0.0
     with pytest.raises(Exception, match="not supported"):
@@ -243,6 +247,9 @@ def test_static_forward_limit_is_checked_on_the_host():
     assert l.mam_fc_forward_static(one, K, one, K, capi.W_MK, None, one, one, one, None, None, N, K, M, None) == -2
     assert b"scratch" in l.mam_last_error()
     assert l.mam_set_option(99, 0) == -1
+    # a value outside the option's range is refused and leaves the option as it was
+    assert l.mam_set_option(capi.OPT_BACKWARD_ONE_LAUNCH, 3) == -1
+    assert l.mam_set_option(capi.OPT_FORWARD_TILING, -1) == -1
     assert l.mam_set_option(capi.OPT_FORWARD_TILING, capi.FORWARD_TILING_AUTO) == 0
 
 

@@ -458,3 +458,21 @@ def test_selected_weights_output(shape):
             capi.fc_forward(x.to(dev), wl.to(dev), layout, x_sel=x_only)
             torch.cuda.synchronize()
         assert torch.equal(x_only, x_sel)
+
+
+def test_nan_products_are_ignored():
+    """NaN products never win and never stick (ordered compares, as in the reference kernel): NaN at k = 0,
+    in mid-row, a whole row of x and a whole weight row, on both tilings, unsplit and with K split."""
+    g = torch.Generator().manual_seed(21)
+    for N, K, M in ((40, 128, 70), (48, 2048, 256)):        # the second shape splits K
+        x = torch.randn(N, K, generator=g)
+        w = torch.randn(M, K, generator=g)
+        x[0, 0] = float("nan")
+        x[1, K // 2 + 3] = float("nan")
+        x[2, :] = float("nan")
+        w[3, :] = float("nan")
+        w[4, 0] = float("nan")
+        w[5, K - 1] = float("nan")
+        x[6, 17] = float("nan")
+        w[6, 17] = float("nan")
+        _run_both_layouts(x, w, None, "nan products %dx%dx%d" % (N, K, M))

@@ -209,6 +209,42 @@ def test_config5_full_size_equals_dense_kernel(density):
     for got_x, got_v in ((xg, vg), (xg2, vg2), (xg3, vg3)):
         assert bool(((got_x - xdg).abs() <= 1e-5 * xdg.abs() + 2.0 ** -21 * xabs).all())
         assert bool(((got_v - want_v).abs() <= 1e-5 * want_v.abs() + 2.0 ** -21 * abs_v).all())
+    # and against the C oracle's CSR backward (fp64 accumulation) over the whole batch, every route
+    amax_c, amin_c = amax.cpu().numpy(), amin.cpu().numpy()
+    want_xg, want_vg = oracle.csr_backward(x.numpy(), crow.numpy(), col.numpy(), val.numpy(), grad.numpy(),
+                                           amax_c, amin_c)
+    floor_xg, floor_vg = oracle.csr_backward(x.abs().numpy(), crow.numpy(), col.numpy(), val.abs().numpy(),
+                                             grad.abs().numpy(), amax_c, amin_c)
+    for route, (got_x, got_v) in (("gather", (xg, vg)), ("w_sel", (xg2, vg2)), ("w_sel + x_sel", (xg3, vg3))):
+        for name, got, want, floor in (("x_grad", got_x, want_xg, floor_xg), ("val_grad", got_v, want_vg, floor_vg)):
+            err = np.abs(got.cpu().numpy().astype(np.float64) - want)
+            bound = 1e-5 * np.abs(want) + 2.0 ** -22 * floor
+            assert (err <= bound).all(), "config 5 %s (%s): worst %.3g over the bound" % (name, route, (err - bound).max())
+
+
+def test_nan_in_stored_values_is_ignored():
+    """A NaN product never wins and never sticks (the dense rule, ordered compares): NaN in a row's first
+    stored value, in mid-row, and a row whose stored values are all NaN (an implicit zero is then both
+    extremes).  x stays finite: the implicit-zero candidate is read at the lowest missing column only."""
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    M, K, N = 48, 200, 70
+    dense, crow, col, val = pruned_csr(M, K, 0.2, seed=9, scale=1.0)
+    val = val.clone()
+    val[crow[0]] = float("nan")
+    val[(crow[1] + crow[2]) // 2] = float("nan")
+    val[crow[2]:crow[3]] = float("nan")
+    val[crow[5] + 1] = float("nan")
+    val[crow[5] + 2] = float("nan")
+    x = torch.randn(N, K, generator=torch.Generator().manual_seed(10))
+    want = oracle.csr_forward(x.numpy(), crow.numpy(), col.numpy(), val.numpy(), K)
+    for n_rows in (N, 33):            # both batch-tile shapes of the kernel
+        c, amax, amin = capi.csr_fc_forward(x[:n_rows].to(dev), crow.to(dev), col.to(dev), val.to(dev), M)
+        torch.cuda.synchronize()
+        assert_bits_equal(c.cpu().numpy(), want[0][:n_rows], "nan values c")
+        assert_index_equal(amax.cpu().numpy(), want[1][:n_rows], "nan values argmax")
+        assert_index_equal(amin.cpu().numpy(), want[2][:n_rows], "nan values argmin")
 
 
 def test_validate_csr_names_what_is_malformed():

@@ -3,6 +3,8 @@ through the operator.  The reference checks it by printing the max-abs error aga
 ``a @ b`` (test/test_sparse.py:33-44); here every cell must be within rtol 1e-5 of the fp64 oracle plus
 the rounding floor of an fp32 sum in any order, 2^-22 x the sum of |terms| of that cell."""
 import numpy as np
+import ctypes
+
 import pytest
 import torch
 
@@ -145,3 +147,56 @@ def test_operator_at_high_density(layout, n, l, m, rate):
     want = a.double() @ b.double()
     floor = a.abs().double() @ b.abs().double()
     assert bool(((res.double() - want).abs() <= 1e-5 * want.abs() + 2.0 ** -22 * floor).all())
+
+
+@pytest.mark.parametrize("layout", [torch.sparse_csr, torch.sparse_coo])
+@pytest.mark.parametrize("above", [False, True])
+def test_operator_either_side_of_the_density_threshold(layout, above):
+    """The operator changes route at one stored entry in eight (sparse kernel below, dense copy + library GEMM
+    from there on), and with it the order of summation: one entry below and exactly at the threshold, both
+    against the fp64 defining sum within rtol 1e-5 plus the rounding floor of an fp32 sum."""
+    R, K, C = 96, 256, 128
+    nnz = R * K // 8 + (0 if above else -1)
+    g = torch.Generator().manual_seed(17 + int(above))
+    where = torch.randperm(R * K, generator=g)[:nnz]
+    a = torch.zeros(R * K)
+    a[where] = torch.randn(nnz, generator=g)
+    a = a.view(R, K).to(DEV)
+    assert int((a != 0).sum()) == nnz
+    b = torch.randn(K, C, generator=g).to(DEV)
+    res = torch.ops.mamtorch_kernel_sparsev1.cusparsemm(a.to_sparse(layout=layout), b)
+    want = a.double() @ b.double()
+    floor = a.abs().double() @ b.abs().double()
+    assert bool(((res.double() - want).abs() <= 1e-5 * want.abs() + 2.0 ** -22 * floor).all())
+
+
+def test_to_dense_skips_coordinates_outside_the_matrix():
+    """mam_csr_to_dense / mam_coo_to_dense write at the coordinates they are given: an entry outside the
+    matrix (a malformed tensor) is dropped instead of written out of range."""
+    R, K = 4, 8
+    crow = torch.tensor([0, 2, 3, 3, 5], dtype=torch.int64, device=DEV)
+    col = torch.tensor([1, 8, -1, 7, 1 << 40], dtype=torch.int64, device=DEV)
+    val = torch.tensor([1.0, 2.0, 3.0, 4.0, 5.0], device=DEV)
+    guard = torch.full((R + 2, K), 9.0, device=DEV)          # rows before and after the matrix must stay
+    from mamtorch_amd import capi
+
+    l = capi.lib()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert l.mam_csr_to_dense(P(crow), P(col), P(val), P(guard[1]), K, R, K, st) == 0
+    torch.cuda.synchronize()
+    want = torch.full((R + 2, K), 9.0)
+    want[1:R + 1] = 0.0
+    want[1, 1] = 1.0
+    want[4, 7] = 4.0
+    assert torch.equal(guard.cpu(), want)
+    row = torch.tensor([0, 4, -1, 3, 2], dtype=torch.int64, device=DEV)
+    col2 = torch.tensor([1, 0, 0, 7, 8], dtype=torch.int64, device=DEV)
+    guard.fill_(9.0)
+    assert l.mam_coo_to_dense(P(row), P(col2), P(val), 5, P(guard[1]), K, R, K, st) == 0
+    torch.cuda.synchronize()
+    want = torch.full((R + 2, K), 9.0)
+    want[1:R + 1] = 0.0
+    want[1, 1] = 1.0
+    want[4, 7] = 4.0
+    assert torch.equal(guard.cpu(), want)

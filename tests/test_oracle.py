@@ -366,3 +366,51 @@ def test_conv_oracle_known_answers_and_cross_checks():
         (yy * gflat).sum().backward()
         assert np.allclose(xg, xt.grad.numpy(), rtol=1e-5, atol=1e-6) and np.allclose(wg, wt.grad.numpy(), rtol=1e-5, atol=1e-6)
         assert L > 0
+
+
+# ---- NaN products: ignored by ordered compares, as by the reference kernel ----
+
+def test_nan_products_known_answers():
+    """Hand-derived.  (1) products [nan, 1, 2]: max 2 at k 2, min 1 at k 1, c = 3.  (2) products
+    [3, nan, -1, nan]: max 3 at 0, min -1 at 2, c = 2.  (3) every product NaN: the extremes keep their
+    starting values -inf / +inf (c = nan) and both indices stay 0.  (4) products [nan, -inf, -inf]: the
+    max never rises above its start, index 0; the min is -inf, first held by k 1."""
+    nan, inf = float("nan"), float("inf")
+    cases = [
+        ([[nan, 1, 2]], [[1], [1], [1]], 3.0, 2, 1),
+        ([[3, 1, -1, 2]], [[1], [nan], [1], [nan]], 2.0, 0, 2),
+        ([[nan, nan]], [[1], [2]], nan, 0, 0),
+        ([[nan, -inf, -inf]], [[1], [1], [1]], -inf, 0, 1),
+    ]
+    for a, b, c_want, imax, imin in cases:
+        a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+        for c, amax, amin in (oracle.forward(a, b), oracle.forward(a, np.ascontiguousarray(b.T), oracle.W_MK),
+                              brute.forward(a, b)):
+            assert_bits_equal(c, np.asarray([[c_want]], np.float32), "nan kat c")
+            assert (int(amax[0, 0]), int(amin[0, 0])) == (imax, imin)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_nan_products_c_scan_equals_brute_force(seed):
+    """The C scan against the pure-Python statement (values sorted out first, index found afterwards) on
+    inputs with NaNs at k = 0, in the middle of rows, in whole rows of x, whole columns of w, and with
+    infinities of both signs."""
+    rng = np.random.default_rng(seed)
+    N, K, M = 7, 19, 6
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    w = rng.standard_normal((M, K)).astype(np.float32)
+    x[0, 0] = np.nan
+    x[1, 7] = np.nan
+    x[2, :] = np.nan
+    w[3, :] = np.nan
+    w[4, 0] = np.nan
+    x[5, 3] = np.inf
+    x[6, 0] = -np.inf
+    w[5, 3] = 0.0                     # inf * 0 = nan
+    with np.errstate(invalid="ignore"):
+        c, amax, amin = oracle.forward(x, w, oracle.W_MK)
+        cb, bmax, bmin = brute.forward(x, np.ascontiguousarray(w.T))
+    assert_bits_equal(c, cb, "nan c")
+    assert_index_equal(amax, bmax, "nan argmax")
+    assert_index_equal(amin, bmin, "nan argmin")
+    assert np.isnan(c[2]).all() and (amax[2] == 0).all() and (amin[:, 3] == 0).all()
