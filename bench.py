@@ -22,8 +22,13 @@ Other workloads (`--workload`), same JSON layout, used for the tables in the des
   sparse_d{10,03,01} 4096x4096 weight pruned to 10 % / 3 % / 1 %, batch 256, CSR forward + backward
   spmm_d{30,10,01}   sum-of-products SpMM (cusparsemm): 4096x4096 CSR with 30 % / 10 % / 1 % stored, times a
                      dense 4096x4096; one op = one multiply-add; torch.sparse.mm timed beside it
+  spmm_sweep         the reference's sparse benchmark grid: sizes 128..4096 x sparse rates 0.7..0.999 x {COO, CSR}
   prune_csr          magnitude pruning of a 4096x4096 weight to 10 % and its compaction to CSR (row offsets +
                      fill); one op = one weight examined; Tensor.to_sparse_csr of the masked weight timed beside it
+  module_headline    the path a user of the reference runs, at the headline shape: mamtorch.nn.FullyConnected(4096,
+                     4096, store_args=True) forward, autograd backward and update_selection_count(); the same
+                     step through the C ABI (pre-allocated outputs) is timed beside it in the same run
+  module_vit_mlp     the same for the two layers of the ViT MLP block (12608 rows, 768 -> 3072 -> 768), no counting
   reference_script   the shape and the operator calls of the reference's own timing loop (test/test.py:186-323):
                      a (128, 2048) x b (2048, 4096) in the reference's (in, out) layout through torch.ops:
                      v1 fullyconnected, v4 fullyconnected, v4 fullyconnected_fast, v4 fullyconnected_backward with
@@ -59,7 +64,7 @@ RAMP_MAX_SECONDS = 3.0
 
 WORKLOADS = ("headline", "config1", "values_headline", "vit_mlp", "inference_m1024", "inference_m4096",
              "inference_m16384", "sparse_d10", "sparse_d03", "sparse_d01", "spmm_d30", "spmm_d10", "spmm_d01", "prune_csr",
-             "reference_script")
+             "reference_script", "module_headline", "module_vit_mlp", "spmm_sweep")
 
 
 class Layer:
@@ -123,6 +128,14 @@ class Layer:
         P = self._p
         rc = self.lib.mam_selection_count(P(self.amax), P(self.amin), P(self.max_count), P(self.min_count),
                                           self.N, self.M, self.K, self.capi.COUNT_HITS, self.sp)
+        assert rc == 0, self.lib.mam_last_error()
+
+    def backward_count(self):
+        P, N, K, M = self._p, self.N, self.K, self.M
+        rc = self.lib.mam_fc_backward_count(P(self.x), K, P(self.w), K, self.capi.W_MK, P(self.g), P(self.amax),
+                                            P(self.amin), P(self.wsel), P(self.xsel), P(self.xg), P(self.wg),
+                                            P(self.max_count), P(self.min_count), self.capi.COUNT_HITS, N, K, M,
+                                            self.sp)
         assert rc == 0, self.lib.mam_last_error()
 
     def describe(self):
@@ -282,11 +295,14 @@ def run_dense(torch, capi, lib, dev, args):
     phases = []
     for i, L in enumerate(layers):
         phases.append(("forward", L.forward))
-    if backward:
-        for L in reversed(layers):
-            phases.append(("backward", L.backward))
-    if count:
-        phases.append(("selection_count", layers[0].count))
+    if backward and count and args.fused_count:
+        phases.append(("backward_and_selection_count", layers[0].backward_count))
+    else:
+        if backward:
+            for L in reversed(layers):
+                phases.append(("backward", L.backward))
+        if count:
+            phases.append(("selection_count", layers[0].count))
     if wl == "headline":
         # one plain 64 MiB copy kernel: the known-size reference that scales the profiler's
         # FETCH_SIZE / WRITE_SIZE counters when traffic is measured
@@ -311,6 +327,17 @@ def run_dense(torch, capi, lib, dev, args):
         out["roofline"]["traffic_source"] = "constant from %s, not measured by this run" % TRAFFIC_PROFILE
         # x, w, c, argmax, argmin and the four hand-over planes (w_sel, x_sel)
         out["roofline"]["algorithmic_bytes"] = 4 * (256 * 4096 + 4096 * 4096 + 8 * 256 * 4096)
+    fused = "backward_and_selection_count" in ph
+    if fused:
+        # one call: x_grad, then w_grad and the counters from the same slabs; the index arrays are read by the
+        # x_grad kernel and once more by the fused kernel (not a third time by a count kernel)
+        L = layers[0]
+        both_ms = ph["backward_and_selection_count"]
+        nbytes = L.backward_bytes() + 4 * 2 * L.M * L.K
+        out["roofline_backward"] = hbm_roofline("mam_bwd_x_kernel + mam_bwd_w_count_kernel (w_grad and hit counts of "
+                                                "the same slabs)", nbytes, both_ms)
+        out["fwd_bwd_count_gops"] = round(triples / ((fwd_ms + both_ms) * 1e-3) / 1e9, 2)
+        backward = count = False
     if backward:
         bwd_ms = ph["backward"]
         out["fwd_bwd_gops"] = round(triples / ((fwd_ms + bwd_ms) * 1e-3) / 1e9, 2)
@@ -466,6 +493,70 @@ def run_spmm(torch, capi, lib, dev, args):
     return ops, ms_step, out, cpu
 
 
+def run_spmm_sweep(torch, capi, lib, dev, args):
+    """spmm_sweep: the reference's own sparse benchmark grid (test/test_sparse.py:51-101, restated): square
+    sizes 128 .. 4096, sparse rates 0.7 .. 0.999, COO and CSR; the operator mamtorch_kernel_sparsev1::cusparsemm
+    on fixed operands, with torch.matmul of the dense operand and torch.sparse.mm beside it (events on the
+    stream; the reference times with the host clock around fresh random operands)."""
+    sizes = [128, 256, 512, 1024, 2048, 4096]
+    rates = [0.7, 0.8, 0.9, 0.95, 0.99, 0.999]
+    layouts = [("coo", torch.sparse_coo), ("csr", torch.sparse_csr)]
+    op = torch.ops.mamtorch_kernel_sparsev1.cusparsemm
+    stream = torch.cuda.current_stream(dev)
+    steps = min(args.steps, 20)
+
+    def timed(fn, reps):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(reps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    # clock ramp on the largest dense product
+    big = torch.randn(4096, 4096, device=dev)
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < RAMP_MIN_SECONDS:
+        big @ big
+        torch.cuda.synchronize()
+    del big
+    cells, total_ops, total_ms = [], 0, 0.0
+    gen = torch.Generator().manual_seed(0)
+    for size in sizes:
+        b = torch.randn(size, size, generator=gen).to(dev)
+        for rate in rates:
+            a = torch.randn(size, size, generator=gen) * torch.bernoulli(torch.full((size, size), 1 - rate), generator=gen)
+            ad = a.to(dev)
+            nnz = int((a != 0).sum())
+            dense_ms = timed(lambda: torch.matmul(ad, b), steps)
+            for name, layout in layouts:
+                asp = ad.to_sparse(layout=layout)
+                ms = timed(lambda: op(asp, b), steps)
+                lib_ms = timed(lambda: torch.sparse.mm(asp, b), max(steps // 4, 3))
+                dense_route = size >= 64 and nnz * 8 >= size * size
+                cells.append({"size": size, "sparse_rate": rate, "layout": name, "nnz": nnz,
+                              "cusparsemm_ms": round(ms, 5), "torch_matmul_dense_ms": round(dense_ms, 5),
+                              "torch_sparse_mm_ms": round(lib_ms, 5),
+                              "route": "densify + at::mm" if dense_route else "%s_spmm_kernel" % name})
+                total_ops += nnz * size
+                total_ms += ms
+    biggest = [c for c in cells if c["size"] == 4096 and c["sparse_rate"] == 0.9 and c["layout"] == "csr"][0]
+    nb = 12 * biggest["nnz"] + 8 * 4096 * 4096
+    out = {
+        "config": {"workload": "sum-of-products SpMM sweep of the reference's sparse benchmark: square sizes %s x "
+                               "sparse rates %s x {COO, CSR}; A = N(0,1) under a Bernoulli mask, b dense N(0,1); "
+                               "one op = one multiply-add of a stored entry; a step = every cell once"
+                               % (sizes, rates), "name": args.workload, "launch": "torch.ops calls"},
+        "cells": cells,
+        "roofline": hbm_roofline("csr_spmm_kernel at 4096, sparse rate 0.9", nb, biggest["cusparsemm_ms"]),
+    }
+    return total_ops, total_ms, out, None
+
+
 def run_prune(torch, capi, lib, dev, args):
     """prune_csr: |w| <= threshold goes (90 % of a N(0, 0.02) weight), survivors compacted to CSR."""
     M = K = 4096
@@ -558,6 +649,102 @@ def run_reference_script(torch, capi, lib, dev, args):
     return triples, ms_step, out, None
 
 
+def run_module(torch, capi, lib, dev, args):
+    """module_headline / module_vit_mlp: nn.FullyConnected modules driven the way a training loop drives them
+    (mamtorch/nn/v4/fullyconnected.py:133-208 forward, mamtorch/kernel/v4/fullyconnected.py:24-41 autograd):
+    forward allocates its outputs, the hand-over planes and the split-K workspace, autograd allocates the
+    gradients.  The C-ABI step over the same operands with pre-allocated buffers runs in the same process."""
+    import mamtorch
+
+    gen = torch.Generator().manual_seed(0)
+    headline = args.workload == "module_headline"
+    if headline:
+        N = 256
+        dims = [(4096, 4096)]
+        text = ("mamtorch.nn.FullyConnected(4096, 4096, bias=True, store_args=True, selection_count_mode='hits') "
+                "at batch 256: forward + autograd backward (grad_x, grad_W, grad_bias) + "
+                "update_selection_count(); x~N(0,1), W~U(-1/64,1/64), grad_out~N(0,1), seed 0")
+    else:
+        N = 12608
+        dims = [(768, 3072), (3072, 768)]
+        text = ("ViT-B/16-shaped MAM MLP block through the module: 12608 rows, nn.FullyConnected 768->3072 and "
+                "3072->768 (bias=True), each fed N(0,1) rows as in the C-ABI workload; forward + autograd backward")
+    layers, shapes = [], []
+    for K, M in dims:
+        layer = mamtorch.nn.FullyConnected(K, M, bias=True, store_args=headline).to(dev).train()
+        if headline:
+            layer.selection_count_mode = "hits"
+        w = (torch.rand(M, K, generator=gen) * 2 - 1) / K ** 0.5
+        x = torch.randn(N, K, generator=gen)
+        g = torch.randn(N, M, generator=gen)
+        with torch.no_grad():
+            layer.weight.copy_(w.to(dev))
+        layers.append(layer)
+        shapes.append((x, w, g))
+    xs = [x.to(dev).requires_grad_(True) for x, _, _ in shapes]
+    gs = [g.to(dev) for _, _, g in shapes]
+    params = [p for layer in layers for p in layer.parameters()]
+    outs = [None] * len(layers)
+
+    def m_forward():
+        for p_ in params:
+            p_.grad = None
+        for x_ in xs:
+            x_.grad = None
+        for i, layer in enumerate(layers):
+            outs[i] = layer(xs[i])
+
+    def m_backward():
+        torch.autograd.backward(outs, gs)
+
+    def m_count():
+        layers[0].update_selection_count()
+
+    phases = [("forward", m_forward), ("backward", m_backward)]
+    if headline:
+        layers[0].reset_selection_count()
+        phases.append(("selection_count", m_count))
+    stream = torch.cuda.current_stream(dev)
+    ms_step, ph = time_phases(torch, stream, phases, args.steps, args.warmup)
+
+    # the same operands through the C ABI, buffers allocated once
+    cl = [Layer(torch, capi, lib, dev, x, layers[i].weight.detach().cpu(), g, True, headline)
+          for i, (x, _, g) in enumerate(shapes)]
+    cph = [("forward", L.forward) for L in cl] + [("backward", L.backward) for L in reversed(cl)]
+    if headline:
+        cph.append(("selection_count", cl[0].count))
+    ms_cabi, ph_cabi = time_phases(torch, stream, cph, args.steps, args.warmup)
+
+    triples = sum(N * K * M for K, M in dims)
+    bwd_bytes = sum(L.backward_bytes() for L in cl)
+    out = {
+        "config": {"workload": text, "name": args.workload,
+                   "layers": [{"N": N, "K": K, "M": M} for K, M in dims],
+                   "launch": "nn.Module forward, torch.autograd.backward, update_selection_count()"},
+        "phases_ms": {k: round(v, 5) for k, v in ph.items()},
+        "forward_gops": round(triples / (ph["forward"] * 1e-3) / 1e9, 2),
+        "c_abi_same_run": {"ms_per_step": round(ms_cabi, 5), "phases_ms": {k: round(v, 5) for k, v in ph_cabi.items()},
+                           "value_gops": round(triples / (ms_cabi * 1e-3) / 1e9, 2)},
+        "module_overhead": {"ms_per_step": round(ms_step - ms_cabi, 5),
+                            "fraction_of_c_abi_step": round((ms_step - ms_cabi) / ms_cabi, 4),
+                            "by_phase_ms": {k: round(ph[k] - ph_cabi[k], 5) for k in ph},
+                            "what": "per step: at::empty of c, argmax, argmin, the (4,N,M) hand-over tensor and the "
+                                    "split-K workspace in the forward; at::empty of both gradients, the bias "
+                                    "gradient (a column sum by ATen) and autograd's bookkeeping in the backward"},
+        "roofline": valu_roofline("; ".join(sorted(set(L.describe() for L in cl))) + " behind the module",
+                                  triples, ph["forward"]),
+        "fwd_bwd_gops": round(triples / ((ph["forward"] + ph["backward"]) * 1e-3) / 1e9, 2),
+        "fwd_bwd_valu_frac": round(3.0 * triples / ((ph["forward"] + ph["backward"]) * 1e-3) / 1e12 / VALU_PEAK_TFLOPS, 4),
+        "roofline_backward": hbm_roofline("mam_bwd_x_kernel + mam_bwd_w_vec_kernel behind autograd (+ bias column sum)",
+                                          bwd_bytes, ph["backward"]),
+    }
+    cpu = None
+    if args.cpu_seconds > 0:
+        cpu = dense_cpu_baseline(torch, [(x, layers[i].weight.detach().cpu(), g) for i, (x, _, g) in enumerate(shapes)],
+                                 args.cpu_seconds, True)
+    return triples, ms_step, out, cpu
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -566,6 +753,8 @@ def main():
                     help="untimed steps after the fixed clock ramp (at least %d phase calls, always run)" % RAMP_MIN_CALLS)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="CPU baseline budget; 0 skips it")
     ap.add_argument("--workload", choices=WORKLOADS, default="headline")
+    ap.add_argument("--fused-count", action="store_true",
+                    help="headline / config1: backward and selection count as ONE call (mam_fc_backward_count)")
     ap.add_argument("--graph", action="store_true",
                     help="dense workloads: record one step into a HIP graph and time replays of it")
     args = ap.parse_args()
@@ -573,7 +762,8 @@ def main():
         print("bench.py measures one GPU: the MAM hot path has no multi-GPU part in this build "
               "(--gpus %d refused)" % args.gpus, file=sys.stderr)
         sys.exit(2)
-    small = args.workload in ("headline", "config1", "values_headline", "prune_csr", "reference_script") \
+    small = args.workload in ("headline", "config1", "values_headline", "prune_csr", "reference_script",
+                              "module_headline") \
         or args.workload.startswith("sparse")
     if args.workload.startswith("spmm"):
         args.steps = 50 if args.steps is None else args.steps
@@ -595,9 +785,11 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     lib = capi.lib()
-    run = run_sparse if args.workload.startswith("sparse") else run_spmm if args.workload.startswith("spmm") \
+    run = run_sparse if args.workload.startswith("sparse") else run_spmm_sweep if args.workload == "spmm_sweep" \
+        else run_spmm if args.workload.startswith("spmm") \
         else run_prune if args.workload == "prune_csr" \
-        else run_reference_script if args.workload == "reference_script" else run_dense
+        else run_reference_script if args.workload == "reference_script" \
+        else run_module if args.workload.startswith("module_") else run_dense
     triples, ms_step, extra, cpu = run(torch, capi, lib, dev, args)
 
     out = {

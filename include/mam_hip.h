@@ -177,6 +177,21 @@ int mam_fc_backward(const float *x, int64_t ldx, const float *w, int64_t ldw, in
                     const float *x_sel, float *x_grad, float *w_grad, int64_t N, int64_t K, int64_t M, void *stream);
 
 /*
+ * mam_fc_backward followed by mam_selection_count(argmax, argmin, max_count, min_count, ..., count_mode) as
+ * ONE call: what a training step does after FullyConnected.forward when the layer keeps selection counts
+ * (mamtorch/kernel/v4/csrc/cuda/fullyconnected_backward.cu:80-135 and then
+ * mamtorch/nn/v4/fullyconnected.py:114-129).  For (M,K) weights, MAM_COUNT_HITS and a batch below 2048 rows the
+ * workgroup that owns four neurons' rows of w_grad also owns their counters: the index arrays are read once
+ * for both and one launch fewer is made; every other case runs the two calls one after the other.  Results
+ * are those of the two calls (w_grad to the same tolerance, counts exact).
+ */
+int mam_fc_backward_count(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                          const float *grad, const int32_t *argmax, const int32_t *argmin,
+                          const float *w_sel, const float *x_sel, float *x_grad, float *w_grad,
+                          int32_t *max_count, int32_t *min_count, int count_mode, int64_t N, int64_t K,
+                          int64_t M, void *stream);
+
+/*
  * The module's `splits` in one call each way (mamtorch/nn/v4/fullyconnected.py:163-176 runs one operator
  * per slice of the input and adds the slices' outputs with ATen).  K is cut into consecutive ranges of
  * `range_len` inputs, the last one shorter; every range is a MAM neuron of its own:

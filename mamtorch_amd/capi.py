@@ -32,7 +32,7 @@ EXPORTS = (
     "mam_fc_forward_static_limit", "mam_fc_forward_static", "mam_fc_forward_describe",
     "mam_fc_forward_workspace", "mam_fc_forward_workspace_for", "mam_fc_forward",
     "mam_fc_forward_values_workspace", "mam_fc_forward_values",
-    "mam_fc_backward", "mam_selection_count",
+    "mam_fc_backward", "mam_fc_backward_count", "mam_selection_count",
     "mam_fc_forward_ranges_workspace", "mam_fc_forward_ranges", "mam_fc_backward_ranges",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward", "mam_csr_validate",
     "mam_csr_spmm", "mam_coo_spmm", "mam_csr_to_dense", "mam_coo_to_dense",
@@ -78,6 +78,8 @@ def lib():
         l.mam_fc_forward_ranges_workspace.argtypes = [_i64, _i64, _i64, _i64, _int]
         l.mam_fc_forward_ranges.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64,
                                             _i64, _ptr, _size, _ptr]
+        l.mam_fc_backward_count.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                            _ptr, _int, _i64, _i64, _i64, _ptr]
         l.mam_fc_backward_ranges.argtypes = [_ptr, _i64, _ptr, _i64, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64,
                                              _i64, _i64, _ptr]
         l.mam_selection_count.argtypes = [_ptr, _ptr, _ptr, _ptr, _i64, _i64, _i64, _int, _ptr]
@@ -196,6 +198,20 @@ def fc_backward(x, w, grad, argmax, argmin, layout=W_KM, want_x=True, want_w=Tru
     with torch.cuda.device(x.device):
         _check(l.mam_fc_backward(_p(x), _ld(x), _p(w), _ld(w), layout, _p(grad), _p(argmax), _p(argmin),
                                  _p(w_sel), _p(x_sel), _p(xg), _p(wg), N, K, M, _stream(x)))
+    return xg, wg
+
+
+def fc_backward_count(x, w, grad, argmax, argmin, max_count, min_count, mode=COUNT_HITS, layout=W_KM, want_x=True,
+                      want_w=True, w_sel=None, x_sel=None):
+    """fc_backward and selection_count (in place on the (M, K) int32 counters) as one call."""
+    l = lib()
+    N, K, M = _dims(x, w, layout)
+    xg = torch.empty((N, K), dtype=torch.float32, device=x.device) if want_x else None
+    wg = torch.empty(tuple(w.shape), dtype=torch.float32, device=x.device) if want_w else None
+    with torch.cuda.device(x.device):
+        _check(l.mam_fc_backward_count(_p(x), _ld(x), _p(w), _ld(w), layout, _p(grad), _p(argmax), _p(argmin),
+                                       _p(w_sel), _p(x_sel), _p(xg), _p(wg), _p(max_count), _p(min_count), mode,
+                                       N, K, M, _stream(x)))
     return xg, wg
 
 

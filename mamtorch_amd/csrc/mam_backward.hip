@@ -22,6 +22,7 @@
 // itself unordered.
 #include "mam_common.h"
 #include "mam_fixed.h"
+#include "mam_count_stream.h"
 
 namespace mam {
 namespace bwd {
@@ -322,11 +323,13 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
 #undef MAM_LOAD_ITEM
 }
 
-// Scatter of one (batch row, 4 consecutive neurons) item into the slab histogram.
-template <int LAYOUT>
+// Scatter of one (batch row, 4 consecutive neurons) item into the slab histogram.  COUNT ((M,K) layout): the
+// picks are also counted in `cnt`, a second LDS plane of the slab's shape whose words hold two 16-bit fields
+// (low: argmax picks, high: argmin picks).
+template <int LAYOUT, bool COUNT = false>
 __device__ __forceinline__ void scatter_quad(float *hist, const float4 &g, const int4 &i1, const int4 &i2,
                                              const float (&x1)[4], const float (&x2)[4], int r0, int k0,
-                                             int kn, int kc, int log2r)
+                                             int kn, int kc, int log2r, uint32_t *cnt = nullptr)
 {
     const float gv[4] = {g.x, g.y, g.z, g.w};
     const int a1[4] = {i1.x - k0, i1.y - k0, i1.z - k0, i1.w - k0};
@@ -334,10 +337,14 @@ __device__ __forceinline__ void scatter_quad(float *hist, const float4 &g, const
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int r = r0 + u;
-        if ((unsigned)a1[u] < (unsigned)kn)
+        if ((unsigned)a1[u] < (unsigned)kn) {
             lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a1[u] : (a1[u] << log2r) + r], x1[u] * gv[u]);
-        if ((unsigned)a2[u] < (unsigned)kn)
+            if (COUNT) atomicAdd(&cnt[r * kc + a1[u]], 1u);
+        }
+        if ((unsigned)a2[u] < (unsigned)kn) {
             lds_add_sparse(&hist[LAYOUT == MAM_W_MK ? r * kc + a2[u] : (a2[u] << log2r) + r], x2[u] * gv[u]);
+            if (COUNT) atomicAdd(&cnt[r * kc + a2[u]], 0x10000u);
+        }
     }
 }
 
@@ -406,14 +413,19 @@ __device__ __forceinline__ void store_slab(const float *hist, float *__restrict_
 // (index load -> gather -> LDS add) overlaps the store phase instead of alternating with it.
 // The work of one workgroup (NT threads) of mam_bwd_w_vec_kernel: workgroup `bx` of `nbx` along the slabs,
 // k chunk `by`, share `bz` of `nbz` of the batch rows.
-template <int LAYOUT, int NT>
+// COUNT: the workgroup also owns the slab's selection counters (hits mode, mam_selcount.hip): the picks it
+// scatters are counted in a second LDS plane behind the histogram and added to max_count / min_count when the
+// slab is streamed out -- the index arrays are read once for both, and one launch serves both.
+template <int LAYOUT, int NT, bool COUNT = false>
 __device__ __forceinline__ void bwd_w_vec_body(
     float *hist, int bx, int nbx, int by, int bz, int nbz,
     const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
     const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
     const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int log2r,
-    int kc, int vec_out, int mtiles, int tiles_per_wg, int rows_per_split, int planes, int range_len)
+    int kc, int vec_out, int mtiles, int tiles_per_wg, int rows_per_split, int planes, int range_len,
+    int32_t *__restrict__ max_count = nullptr, int32_t *__restrict__ min_count = nullptr)
 {
+    uint32_t *cnt = reinterpret_cast<uint32_t *>(hist) + ((size_t)kc << log2r);
     const int tid = threadIdx.x;
     const int R = 1 << log2r;
     const int qpr = R >> 2;
@@ -464,10 +476,10 @@ __device__ __forceinline__ void bwd_w_vec_body(
         const int rn = (M - m0) < R ? (M - m0) : R;
         float x1[4] = {s1.x, s1.y, s1.z, s1.w}, x2[4] = {s2.x, s2.y, s2.z, s2.w};
         if (have && !x_sel) gather_quad(x + (int64_t)n_first * ldx + k0, i1, i2, k0, kn, x1, x2);
-        for (int i = tid * 4; i < R * kc; i += NT * 4)
+        for (int i = tid * 4; i < (COUNT ? 2 : 1) * R * kc; i += NT * 4)
             *reinterpret_cast<float4 *>(&hist[i]) = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
-        if (have) scatter_quad<LAYOUT>(hist, g, i1, i2, x1, x2, r_first, k0, kn, kc, log2r);
+        if (have) scatter_quad<LAYOUT, COUNT>(hist, g, i1, i2, x1, x2, r_first, k0, kn, kc, log2r, cnt);
         for (int64_t it = tid + NT; it < items; it += NT) {
             const int pl = npl > 1 ? (int)(it / per_plane) : 0;
             const int64_t rem = npl > 1 ? it - pl * per_plane : it;
@@ -487,10 +499,14 @@ __device__ __forceinline__ void bwd_w_vec_body(
             } else {
                 gather_quad(x + (int64_t)n * ldx + k0, j1, j2, k0, kn, y1, y2);
             }
-            scatter_quad<LAYOUT>(hist, gg, j1, j2, y1, y2, r0, k0, kn, kc, log2r);
+            scatter_quad<LAYOUT, COUNT>(hist, gg, j1, j2, y1, y2, r0, k0, kn, kc, log2r, cnt);
         }
         __syncthreads();
         if (t + 1 < tiles_per_wg && mt + 1 < mtiles) load_first(m0 + R);
+        // the counters first: their read-modify-write is the longer chain, the plain stores of w_grad follow it
+        // (measured at 256 x 4096 x 4096, x_grad + this kernel: 58.7 us this way round, 61.2 the other)
+        if (COUNT)
+            selcount::stream_counts<MAM_COUNT_HITS, NT, 2>(cnt, max_count, min_count, tid, m0, k0, rn, kn, kc, K);
         store_slab<LAYOUT, NT>(hist, w_grad, tid, m0, k0, rn, kn, kc, log2r, K, M, vec_out, accumulate);
         __syncthreads();
     }
@@ -507,6 +523,146 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_w_vec_kernel(
     bwd_w_vec_body<LAYOUT, NT_W>(hist, blockIdx.x, gridDim.x, blockIdx.y, blockIdx.z, gridDim.z, x, ldx, grad, argmax,
                                  argmin, x_sel, nm, w_grad, N, K, M, log2r, kc, vec_out, mtiles, tiles_per_wg,
                                  rows_per_split, planes, range_len);
+}
+
+// w_grad and the selection counts (hits) of the same slabs in one launch.
+constexpr int NT_C = 1024;   // both LDS planes of a slab are 128 KiB: one workgroup per CU, so twice the threads
+__global__ __launch_bounds__(NT_C) void mam_bwd_w_count_kernel(
+    const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
+    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
+    const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int32_t *__restrict__ max_count,
+    int32_t *__restrict__ min_count, int N, int K, int M, int log2r, int kc, int mtiles, int tiles_per_wg)
+{
+    extern __shared__ float hist[];
+    bwd_w_vec_body<MAM_W_MK, NT_C, true>(hist, blockIdx.x, gridDim.x, blockIdx.y, 0, 1, x, ldx, grad, argmax, argmin,
+                                         x_sel, nm, w_grad, N, K, M, log2r, kc, 1, mtiles, tiles_per_wg, N, 1, K,
+                                         max_count, min_count);
+}
+
+// w_grad as the exact sum of its fp32 terms, rounded once (option MAM_OPT_BACKWARD_EXACT; (M,K) weights, 16-byte
+// aligned operands).  A workgroup owns 4 neurons x kc columns in 64-bit fixed-point cells (mam_fixed.h): integer
+// adds are exact and commute, so w_grad does not depend on the order in which the lanes arrive and equals the
+// correctly rounded sum.  An 8-byte cell halves the columns a 64 KiB slab holds, so a neuron quad with K = 4096
+// is covered by two workgroups that each scan the quad's items: 32 against 17 us at 256 x 4096 x 4096, which is
+// why this is an option and not the default.  Terms outside the window (more than ~2^25 below the largest, inf,
+// nan) go through the queue and are added in fp64 before the one rounding; if more than QCAP terms of a
+// workgroup fall outside, that workgroup falls back to fp32 LDS atomics (and its cells are then sums in arrival
+// order, within the documented tolerance).
+constexpr int NT_E = 1024;
+__global__ __launch_bounds__(NT_E) void mam_bwd_w_exact_kernel(
+    const float *__restrict__ x, int64_t ldx, const float *__restrict__ grad,
+    const int32_t *__restrict__ argmax, const int32_t *__restrict__ argmin,
+    const float *__restrict__ x_sel, int64_t nm, float *__restrict__ w_grad, int N, int K, int M, int kc, int span)
+{
+    using namespace fixedpoint;
+    extern __shared__ unsigned long long exact_cells[];      // [4][kc]
+    __shared__ FixedQueue q;
+    __shared__ uint32_t s_max;
+    float *hist = reinterpret_cast<float *>(exact_cells);
+    const int tid = threadIdx.x;
+    const int m0 = xcd_remap(blockIdx.x, gridDim.x) * 4;
+    const int k0 = blockIdx.y * kc;
+    const int kn = (K - k0) < kc ? (K - k0) : kc;
+    const int ncells = 4 * kc;
+
+    // one item: batch row n, neurons m0 .. m0 + 3; cell index per term, -1 = outside this k chunk
+    float t1[4], t2[4];
+    int c1[4], c2[4];
+    auto load_item = [&](int n) {
+        const int64_t o = (int64_t)n * M + m0;
+        const float4 g = *reinterpret_cast<const float4 *>(grad + o);
+        const int4 i1 = *reinterpret_cast<const int4 *>(argmax + o);
+        const int4 i2 = *reinterpret_cast<const int4 *>(argmin + o);
+        const float gv[4] = {g.x, g.y, g.z, g.w};
+        const int a1[4] = {i1.x - k0, i1.y - k0, i1.z - k0, i1.w - k0};
+        const int a2[4] = {i2.x - k0, i2.y - k0, i2.z - k0, i2.w - k0};
+        float x1[4], x2[4];
+        if (x_sel) {
+            const float4 s1 = *reinterpret_cast<const float4 *>(x_sel + o);
+            const float4 s2 = *reinterpret_cast<const float4 *>(x_sel + nm + o);
+            x1[0] = s1.x; x1[1] = s1.y; x1[2] = s1.z; x1[3] = s1.w;
+            x2[0] = s2.x; x2[1] = s2.y; x2[2] = s2.z; x2[3] = s2.w;
+        } else {
+            const float *xr = x + (int64_t)n * ldx + k0;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                x1[u] = (unsigned)a1[u] < (unsigned)kn ? xr[a1[u]] : 0.0f;
+                x2[u] = (unsigned)a2[u] < (unsigned)kn ? xr[a2[u]] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            c1[u] = (unsigned)a1[u] < (unsigned)kn ? u * kc + a1[u] : -1;
+            c2[u] = (unsigned)a2[u] < (unsigned)kn ? u * kc + a2[u] : -1;
+            t1[u] = x1[u] * gv[u];
+            t2[u] = x2[u] * gv[u];
+        }
+    };
+
+    if (tid == 0) {
+        s_max = 0u;
+        q.count = 0;
+    }
+    __syncthreads();
+    bool fixed = span >= 8;
+    bool loaded = false;
+    int e_lo = 1;
+    if (fixed) {
+        uint32_t mx = 0u;
+        if (tid < N) {
+            load_item(tid);
+            loaded = true;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (c1[u] >= 0) { const uint32_t b = magnitude_bits(t1[u]); mx = mx > b ? mx : b; }
+                if (c2[u] >= 0) { const uint32_t b = magnitude_bits(t2[u]); mx = mx > b ? mx : b; }
+            }
+        }
+        fixed = make_window(workgroup_max(mx, &s_max), N <= NT_E ? 0 : 4, span, e_lo);
+    }
+    for (int attempt = fixed ? 0 : 1; attempt < 2; ++attempt) {
+        const bool fx = attempt == 0;
+        if (fx) for (int i = tid; i < ncells; i += NT_E) exact_cells[i] = 0ull;
+        else for (int i = tid; i < ncells; i += NT_E) hist[i] = 0.0f;
+        __syncthreads();
+        for (int n = tid; n < N; n += NT_E) {
+            if (!loaded) load_item(n);
+            loaded = false;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (c1[u] >= 0) {
+                    if (!fx) lds_add_sparse(&hist[c1[u]], t1[u]);
+                    else if (fixed_add(&exact_cells[c1[u]], t1[u], e_lo, span)) queue_push(q, c1[u], t1[u]);
+                }
+                if (c2[u] >= 0) {
+                    if (!fx) lds_add_sparse(&hist[c2[u]], t2[u]);
+                    else if (fixed_add(&exact_cells[c2[u]], t2[u], e_lo, span)) queue_push(q, c2[u], t2[u]);
+                }
+            }
+        }
+        __syncthreads();
+        const int queued = fx ? q.count : 0;
+        __syncthreads();
+        if (queued > QCAP) {
+            if (tid == 0) q.count = 0;
+            continue;      // the window was a bad guess: once more with fp32 atomics
+        }
+        if (queued > 0) settle_queue<NT_E>(exact_cells, ncells, q, queued, e_lo, 0);
+        const double *d = reinterpret_cast<const double *>(exact_cells);
+        const int q4 = kn >> 2;
+        for (int e = tid; e < 4 * q4; e += NT_E) {
+            const int r = e / q4, c4 = (e - r * q4) * 4;
+            if (m0 + r >= M) continue;
+            float4 v;
+            const int b = r * kc + c4;
+            if (queued > 0) v = make_float4((float)d[b], (float)d[b + 1], (float)d[b + 2], (float)d[b + 3]);
+            else if (fx) v = make_float4(cell_value(exact_cells[b], e_lo), cell_value(exact_cells[b + 1], e_lo),
+                                         cell_value(exact_cells[b + 2], e_lo), cell_value(exact_cells[b + 3], e_lo));
+            else v = make_float4(hist[b], hist[b + 1], hist[b + 2], hist[b + 3]);
+            *reinterpret_cast<float4 *>(w_grad + (int64_t)(m0 + r) * K + k0 + c4) = v;
+        }
+        break;
+    }
 }
 
 // Both gradients in one launch, for the shapes where one launch of each kind fills the chip once: the first
@@ -602,7 +758,7 @@ static int setup_device(int dev)
         (const void *)mam_bwd_x_kernel<MAM_W_MK>,      (const void *)mam_bwd_x_kernel<MAM_W_KM>,
         (const void *)mam_bwd_w_kernel<MAM_W_MK>,      (const void *)mam_bwd_w_kernel<MAM_W_KM>,
         (const void *)mam_bwd_w_vec_kernel<MAM_W_MK>,  (const void *)mam_bwd_w_vec_kernel<MAM_W_KM>,
-        (const void *)mam_bwd_both_kernel<MAM_W_MK>,
+        (const void *)mam_bwd_both_kernel<MAM_W_MK>,   (const void *)mam_bwd_w_count_kernel,
     };
     bool all = true;
     for (const void *k : kernels)
@@ -663,6 +819,19 @@ static int launch_layout(const float *x, int64_t ldx, const float *w, int64_t ld
         // a quarter of every 64-byte sector it touches.  When K is small enough, 16 neurons (whole
         // sectors) share a slab, and the batch is split over several workgroups per slab to keep the
         // chip filled; they add their shares to the cleared w_grad.
+        if (LAYOUT == MAM_W_MK && vec_in && planes == 1 && K % 4 == 0 && (uintptr_t)w_grad % 16 == 0 &&
+            option(MAM_OPT_BACKWARD_EXACT) == MAM_BACKWARD_EXACT_ON) {
+            // 4 neurons x kc columns of 8-byte cells in 64 KiB
+            int kce = 2048;
+            if (K < kce) kce = (int)K;
+            const int64_t kt = ceil_div(K, kce);
+            if (kt <= 65535) {
+                hipLaunchKernelGGL(mam_bwd_w_exact_kernel, dim3((unsigned)(M / 4), (unsigned)kt), dim3(NT_E),
+                                   (size_t)4 * kce * 8, st, x, ldx, grad, argmax, argmin, x_sel, N * M, w_grad, (int)N,
+                                   (int)K, (int)M, kce, window_span(2 * N));
+                return check_launch("mam_bwd_w_exact_kernel");
+            }
+        }
         const bool large_batch = LAYOUT == MAM_W_MK && vec_in && N >= 2048;
         if (large_batch)
             while (log2r < 4 && ((int64_t)2 << log2r) * ((K + 3) / 4 * 4) * 4 <= 64 * 1024) ++log2r;
@@ -757,6 +926,42 @@ static int launch_both(const float *x, int64_t ldx, const float *w, int64_t ldw,
     return check_launch("mam_bwd_both_kernel");
 }
 
+// w_grad and the hits-mode selection counts in one launch (mam_bwd_w_count_kernel) where the shape allows it:
+// (M,K) weights, the 16-byte paths, a batch below the large-batch shapes and below 32768 rows (16-bit count
+// fields), both LDS planes of a slab within the device's limit.  Returns 1 when the shape is not served.
+static int launch_w_count(const float *x, int64_t ldx, const float *grad, const int32_t *argmax,
+                          const int32_t *argmin, const float *x_sel, float *w_grad, int32_t *max_count,
+                          int32_t *min_count, int64_t N, int64_t K, int64_t M, hipStream_t st)
+{
+    const int dev = ensure_device(st);
+    if (dev < 0) return dev;
+    const bool vec = (M % 4 == 0) && (N * M % 4 == 0) && (K % 4 == 0) && ((uintptr_t)grad % 16 == 0) &&
+                     ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)x_sel % 16 == 0) &&
+                     ((uintptr_t)w_grad % 16 == 0) && ((uintptr_t)max_count % 16 == 0) &&
+                     ((uintptr_t)min_count % 16 == 0);
+    if (!vec || N >= 2048 || N >= 32768) return 1;
+    const int log2r = 2, R = 4;
+    // histogram + count plane of a slab: 4 neurons x kc columns x 8 bytes
+    const int64_t lds_cap_bytes = (int64_t)g_lds_floats[dev] * 4;
+    // whole rows of K = 4096 (one workgroup per CU); half rows with two workgroups per CU read the index
+    // arrays twice and took 71 against 59 us at 256 x 4096 x 4096
+    int64_t kc = 4096;
+    while (kc > 64 && (int64_t)R * kc * 8 > lds_cap_bytes) kc /= 2;
+    if (K < kc) kc = (K + 3) / 4 * 4;
+    if ((int64_t)R * kc * 8 > lds_cap_bytes) return 1;
+    const int64_t mtiles = ceil_div(M, R), ktiles = ceil_div(K, kc);
+    if (ktiles > 65535) return 1;
+    const int cus = num_cus();
+    const int64_t per_cu = (160 * 1024) / (R * kc * 8) < 1 ? 1 : (160 * 1024) / (R * kc * 8);
+    int tpw = (int)(mtiles * ktiles / (per_cu * cus));
+    if (tpw < 1) tpw = 1;
+    if (tpw > 8) tpw = 8;
+    hipLaunchKernelGGL(mam_bwd_w_count_kernel, dim3((unsigned)ceil_div(mtiles, tpw), (unsigned)ktiles), dim3(NT_C),
+                       (size_t)R * kc * 8, st, x, ldx, grad, argmax, argmin, x_sel, N * M, w_grad, max_count, min_count,
+                       (int)N, (int)K, (int)M, log2r, (int)kc, (int)mtiles, tpw);
+    return check_launch("mam_bwd_w_count_kernel");
+}
+
 // x_grad from selected weights handed over by a forward, whatever that forward read them from.
 int x_grad_from_selected(const float *grad, const int32_t *argmax, const int32_t *argmin, const float *w_sel,
                          float *x_grad, int64_t N, int64_t K, int64_t M, hipStream_t st)
@@ -806,7 +1011,8 @@ static int backward_impl(const float *x, int64_t ldx, const float *w, int64_t ld
     // x_grad is bound by LDS atomics and w_grad by memory traffic, and neither depends on the other: one
     // launch that holds both where the shape allows it, else two streams where that pays
     if (x_grad && w_grad && w_layout == MAM_W_MK && option(MAM_OPT_BACKWARD_ONE_LAUNCH) != MAM_BACKWARD_ONE_LAUNCH_OFF &&
-        option(MAM_OPT_BACKWARD_FORK) != MAM_BACKWARD_FORK_ON) {
+        option(MAM_OPT_BACKWARD_FORK) != MAM_BACKWARD_FORK_ON &&
+        option(MAM_OPT_BACKWARD_EXACT) != MAM_BACKWARD_EXACT_ON) {
         const int rc = bwd::launch_both(x, ldx, w, ldw, grad, argmax, argmin, w_sel, x_sel, x_grad, w_grad, N, K, M, st,
                                         planes, range_len,
                                         option(MAM_OPT_BACKWARD_ONE_LAUNCH) == MAM_BACKWARD_ONE_LAUNCH_AUTO);
@@ -832,6 +1038,37 @@ extern "C" int mam_fc_backward(const float *x, int64_t ldx, const float *w, int6
 {
     return backward_impl(x, ldx, w, ldw, w_layout, grad, argmax, argmin, w_sel, x_sel, x_grad, w_grad, N, K, M, 1, 0,
                          stream);
+}
+
+extern "C" int mam_fc_backward_count(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,
+                                     const float *grad, const int32_t *argmax, const int32_t *argmin,
+                                     const float *w_sel, const float *x_sel, float *x_grad, float *w_grad,
+                                     int32_t *max_count, int32_t *min_count, int count_mode, int64_t N, int64_t K,
+                                     int64_t M, void *stream)
+{
+    using namespace mam;
+    if (count_mode != MAM_COUNT_REFERENCE && count_mode != MAM_COUNT_HITS && count_mode != MAM_COUNT_FLAGS)
+        return fail(MAM_ERR_INVALID_ARGUMENT, "unknown selection-count mode %d", count_mode);
+    if (!max_count || (count_mode != MAM_COUNT_REFERENCE && !min_count))
+        return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    // the fused kernel: every operand of the plain calls valid, (M,K) weights, hits, w_grad wanted
+    const bool fusable = count_mode == MAM_COUNT_HITS && w_layout == MAM_W_MK && w_grad && x && w && grad && argmax &&
+                         argmin && N > 0 && M > 0 && K > 0 && N <= INT32_MAX / 2 && K <= INT32_MAX / 2 &&
+                         M <= INT32_MAX / 2 && ldx >= K && ldw >= K;
+    if (fusable) {
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        const int rc_w = bwd::launch_w_count(x, ldx, grad, argmax, argmin, x_sel, w_grad, max_count, min_count, N, K, M,
+                                             st);
+        if (rc_w != 1) {
+            if (rc_w != MAM_OK || !x_grad) return rc_w;
+            return backward_impl(x, ldx, w, ldw, w_layout, grad, argmax, argmin, w_sel, x_sel, x_grad, nullptr, N, K, M,
+                                 1, 0, stream);
+        }
+    }
+    const int rc = backward_impl(x, ldx, w, ldw, w_layout, grad, argmax, argmin, w_sel, x_sel, x_grad, w_grad, N, K, M, 1,
+                                 0, stream);
+    if (rc != MAM_OK) return rc;
+    return mam_selection_count(argmax, argmin, max_count, min_count, N, M, K, count_mode, stream);
 }
 
 extern "C" int mam_fc_backward_ranges(const float *x, int64_t ldx, const float *w, int64_t ldw, int w_layout,

@@ -18,6 +18,7 @@
 // the literal rule of the retired convolution modules (mamtorch/nn/backup/mamconv1d.txt:84-103), whose two
 // advanced-index "+= 1" statements write the two counters.
 #include "mam_common.h"
+#include "mam_count_stream.h"
 
 namespace mam {
 namespace selcount {
@@ -91,54 +92,7 @@ __global__ __launch_bounds__(NT_H) void count_kernel(const int32_t *__restrict__
         // them was hit.  At training batch sizes nearly every cache line holds a hit, so this is
         // a coalesced read-modify-write of the slab; at small N*M it degenerates to a sparse one.
         if (vec) {
-            const int q = kn >> 2;
-            const int total = rn * q;
-            for (int eb = tid; eb < total; eb += FU * NT_H) {
-                uint4 v[FU];
-                int4 amx[FU], amn[FU];
-                int64_t cell[FU];
-#pragma unroll
-                for (int u = 0; u < FU; ++u) {
-                    const int e = eb + u * NT_H;
-                    v[u] = make_uint4(0u, 0u, 0u, 0u);
-                    cell[u] = 0;
-                    if (e < total) {
-                        const int r = e / q, c4 = e - r * q;
-                        v[u] = *reinterpret_cast<const uint4 *>(&cnt[r * kc + c4 * 4]);
-                        cell[u] = (int64_t)(m0 + r) * K + k0 + c4 * 4;
-                    }
-                }
-                if (MODE == MAM_COUNT_REFERENCE) {
-                    // both flags land in max_count: fold them into the low field
-#pragma unroll
-                    for (int u = 0; u < FU; ++u) {
-                        v[u].x = (v[u].x & 1u) + (v[u].x >> 16);
-                        v[u].y = (v[u].y & 1u) + (v[u].y >> 16);
-                        v[u].z = (v[u].z & 1u) + (v[u].z >> 16);
-                        v[u].w = (v[u].w & 1u) + (v[u].w >> 16);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < FU; ++u) {
-                    const uint32_t any = v[u].x | v[u].y | v[u].z | v[u].w;
-                    if (any & 0xffffu) amx[u] = *reinterpret_cast<const int4 *>(max_count + cell[u]);
-                    if (any >> 16) amn[u] = *reinterpret_cast<const int4 *>(min_count + cell[u]);
-                }
-#pragma unroll
-                for (int u = 0; u < FU; ++u) {
-                    const uint32_t any = v[u].x | v[u].y | v[u].z | v[u].w;
-                    if (any & 0xffffu) {
-                        amx[u].x += (int)(v[u].x & 0xffffu); amx[u].y += (int)(v[u].y & 0xffffu);
-                        amx[u].z += (int)(v[u].z & 0xffffu); amx[u].w += (int)(v[u].w & 0xffffu);
-                        *reinterpret_cast<int4 *>(max_count + cell[u]) = amx[u];
-                    }
-                    if (any >> 16) {
-                        amn[u].x += (int)(v[u].x >> 16); amn[u].y += (int)(v[u].y >> 16);
-                        amn[u].z += (int)(v[u].z >> 16); amn[u].w += (int)(v[u].w >> 16);
-                        *reinterpret_cast<int4 *>(min_count + cell[u]) = amn[u];
-                    }
-                }
-            }
+            stream_counts<MODE, NT_H, FU>(cnt, max_count, min_count, tid, m0, k0, rn, kn, kc, K);
         } else {
             for (int e = tid; e < rn * kn; e += NT_H) {
                 const int r = e / kn, kk = e - r * kn;

@@ -32,11 +32,14 @@ def register_exact_forward(ns):
         _, argmax, argmin = output
         need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         ctx.save_for_backward(a if need else None, b if need else None, argmax, argmin)
+        # the index outputs never receive a gradient: without this autograd fills two (N, out) tensors with
+        # zeros for them before every backward
+        ctx.set_materialize_grads(False)
 
     def _backward(ctx, grad):
         a, b, argmax, argmin = ctx.saved_tensors
         a_grad, b_grad = None, None
-        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+        if grad[0] is not None and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]):
             a_grad, b_grad = ops.fullyconnected_backward.default(a, b, grad[0].contiguous(), argmax, argmin)
         return a_grad, b_grad
 

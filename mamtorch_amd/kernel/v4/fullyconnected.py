@@ -69,12 +69,17 @@ def _wt_setup_context(ctx, inputs, output):
     need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
     ctx.save_for_backward(a if need else None, weight if need else None, argmax, argmin,
                           sel if need else None)
+    # argmax, argmin and the hand-over tensor never receive a gradient: without this autograd fills three
+    # tensors (2 x (N, out) int32 and (4, N, out) fp32) with zeros before every backward
+    ctx.set_materialize_grads(False)
 
 
 def _wt_backward(ctx, grad):
     a, weight, argmax, argmin, sel = ctx.saved_tensors
     a_grad, w_grad, bias_grad = None, None, None
     g = grad[0]
+    if g is None:
+        return None, None, None, None
     if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
         a_grad, w_grad = K.fullyconnected_wt_backward.default(a, weight, g.contiguous(), argmax, argmin, sel)
     if ctx.needs_input_grad[2]:

@@ -43,12 +43,15 @@ def _ranges_setup(ctx, inputs, output):
     need = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
     ctx.range_len, ctx.with_indices = range_len, with_indices
     ctx.save_for_backward(a if need else None, weight if need else None, argmax, argmin)
+    ctx.set_materialize_grads(False)      # no zero-filled gradients for the index outputs
 
 
 def _ranges_backward(ctx, grad):
     a, weight, argmax, argmin = ctx.saved_tensors
     a_grad = w_grad = bias_grad = None
     g = grad[0]
+    if g is None:
+        return None, None, None, None, None
     if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
         if not ctx.with_indices:
             raise RuntimeError("fullyconnected_ranges was run without indices; its gradient needs them")

@@ -347,3 +347,115 @@ def test_x_grad_is_reproducible_bit_for_bit(shape):
     assert torch.equal(first, gathered)
     gathered, _ = capi.fc_backward(xd, wd.T.contiguous(), gd, amax, amin, capi.W_KM, want_w=False)
     assert torch.equal(first, gathered)
+
+
+# ---- strict gradient parity: option MAM_OPT_BACKWARD_EXACT ----
+
+def _exact_gradients(x, w, grad, with_x_sel=True):
+    """Forward with the hand-over, then the backward with w_grad in fixed-point cells: (x_grad, w_grad,
+    oracle x_grad, oracle w_grad) as numpy arrays."""
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    N, M = x.shape[0], w.shape[0]
+    xd, wd, gd = x.to(dev), w.to(dev), grad.to(dev)
+    ws = torch.empty(2, N, M, device=dev)
+    xs = torch.empty(2, N, M, device=dev)
+    _, amax, amin = capi.fc_forward(xd, wd, capi.W_MK, w_sel=ws, x_sel=xs)
+    capi.set_option(capi.OPT_BACKWARD_EXACT, 1)
+    try:
+        xg, wg = capi.fc_backward(xd, wd, gd, amax, amin, capi.W_MK, w_sel=ws, x_sel=xs if with_x_sel else None)
+        torch.cuda.synchronize()
+    finally:
+        capi.set_option(capi.OPT_BACKWARD_EXACT, 0)
+    xo, wo = oracle.backward(x.numpy(), w.numpy(), grad.numpy(), amax.cpu().numpy(), amin.cpu().numpy(), oracle.W_MK)
+    return xg.cpu().numpy(), wg.cpu().numpy(), xo, wo
+
+
+@pytest.mark.parametrize("config", ["config 1", "config 2"])
+@pytest.mark.parametrize("with_x_sel", [True, False])
+def test_exact_option_gradients_equal_the_oracle_bit_for_bit(config, with_x_sel):
+    """With MAM_OPT_BACKWARD_EXACT both gradients are exact sums of their fp32 terms rounded once: bit-equal
+    to the oracle's fp64-accumulated values at the two configurations the CPU oracle runs whole, no
+    tolerance, no summation floor."""
+    if config == "config 1":
+        x, w, _, grad = config1()
+    else:
+        g = torch.Generator().manual_seed(0)
+        x = torch.randn(256, 4096, generator=g)
+        w = (torch.rand(4096, 4096, generator=g) * 2 - 1) / 64
+        grad = torch.randn(256, 4096, generator=g)
+    xg, wg, xo, wo = _exact_gradients(x, w, grad, with_x_sel)
+    assert np.array_equal(xg.view(np.int32), xo.view(np.int32)), config + ": x_grad is not the rounded exact sum"
+    assert np.array_equal(wg.view(np.int32), wo.view(np.int32)), config + ": w_grad is not the rounded exact sum"
+
+
+@pytest.mark.parametrize("dims", [(768, 3072), (3072, 768)])
+def test_exact_option_meets_plain_rtol_at_config3(dims):
+    """Config 3 (12608 rows) with MAM_OPT_BACKWARD_EXACT: plain rtol 1e-5 on every cell of both gradients,
+    no floor term (cells whose terms cancel included)."""
+    K, M = dims
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(12608, K, generator=g)
+    w = (torch.rand(M, K, generator=g) * 2 - 1) / K ** 0.5
+    grad = torch.randn(12608, M, generator=g)
+    xg, wg, xo, wo = _exact_gradients(x, w, grad)
+    for name, got, want in (("x_grad", xg, xo), ("w_grad", wg, wo)):
+        err = np.abs(got.astype(np.float64) - want)
+        assert (err <= RTOL * np.abs(want)).all(), "config 3 %s: worst %.3g relative" % (
+            name, (err[want != 0] / np.abs(want[want != 0])).max())
+
+
+def test_exact_option_on_ragged_and_small_shapes():
+    """Shapes the fixed-point w_grad kernel serves (M and K multiples of 4) with a partial last k chunk, and
+    shapes it does not serve, which fall through to the fp32 route: all within the documented bar."""
+    from mamtorch_amd import capi
+
+    capi.set_option(capi.OPT_BACKWARD_EXACT, 1)
+    try:
+        for shape in ((33, 2052, 8), (5, 4, 4), (300, 4100, 12), (17, 9, 300), (64, 784, 256)):
+            x, w, grad = random_case(*shape, seed=sum(shape))
+            _, amax, amin = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+            _check(x, w, grad, amax, amin, "exact option, shape %s" % (shape,))
+    finally:
+        capi.set_option(capi.OPT_BACKWARD_EXACT, 0)
+
+
+# ---- backward and selection count in one call ----
+
+@pytest.mark.parametrize("shape", [(256, 4096, 4096), (64, 784, 256), (300, 1028, 36), (33, 100, 18), (2100, 64, 8)])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_backward_count_equals_the_two_calls(shape, mode):
+    """mam_fc_backward_count = mam_fc_backward followed by mam_selection_count: counts exactly equal, x_grad
+    bit-equal (the same kernel), w_grad equal within the documented bar (the fused kernel adds in another
+    order).  Shapes on and off the fused route, every count mode, counters that are not zero at the start."""
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    N, K, M = shape
+    x, w, grad = random_case(N, K, M, seed=N + mode)
+    xd, wd, gd = x.to(dev), w.to(dev), grad.to(dev)
+    ws = torch.empty(2, N, M, device=dev)
+    xs = torch.empty(2, N, M, device=dev)
+    _, amax, amin = capi.fc_forward(xd, wd, capi.W_MK, w_sel=ws, x_sel=xs)
+    start = torch.randint(0, 5, (M, K), dtype=torch.int32, generator=torch.Generator().manual_seed(1)).to(dev)
+    mc1, nc1, mc2, nc2 = start.clone(), start.clone(), start.clone(), start.clone()
+    xg1, wg1 = capi.fc_backward(xd, wd, gd, amax, amin, capi.W_MK, w_sel=ws, x_sel=xs)
+    capi.selection_count(amax, amin, mc1, nc1, mode)
+    xg2, wg2 = capi.fc_backward_count(xd, wd, gd, amax, amin, mc2, nc2, mode, capi.W_MK, w_sel=ws, x_sel=xs)
+    torch.cuda.synchronize()
+    assert torch.equal(mc1, mc2) and torch.equal(nc1, nc2)
+    assert torch.equal(xg1, xg2)
+    _, wabs = capi.fc_backward(xd.abs(), wd.abs(), gd.abs(), amax, amin, capi.W_MK, want_x=False)
+    torch.cuda.synchronize()
+    assert bool(((wg1 - wg2).abs() <= 2 * (RTOL * wg1.abs() + FLOOR * wabs)).all())
+    # and the counts against the oracle
+    before = start.cpu().numpy()
+    if mode == 2:     # flags, max and min apart: +1 where at least one batch row picked the cell
+        want_m, want_n = before.copy(), before.copy()
+        cols = np.broadcast_to(np.arange(M), (N, M))
+        want_m[cols, amax.cpu().numpy()] += 1
+        want_n[cols, amin.cpu().numpy()] += 1
+    else:
+        want_m, want_n = oracle.selection_count(amax.cpu().numpy(), amin.cpu().numpy(), before, before, mode=mode)
+    assert np.array_equal(mc2.cpu().numpy(), want_m) and np.array_equal(nc2.cpu().numpy(), want_n)
