@@ -350,6 +350,29 @@ int mam_prune_fill_csr(const float *w, int64_t ldw, int mode, const void *aux, c
 int mam_prune_apply(float *w, int64_t ldw, int mode, const void *aux, const void *aux2, int64_t ld_aux,
                     float threshold, int64_t M, int64_t K, void *stream);
 
+/*
+ * The pruning threshold without a sort: the element(s) of given rank among the absolute scores of one or
+ * several matrices.  Replaces `torch.quantile(flattened_weights.abs(), p)`
+ * (examples/vitb16_imagenet1k/pruning_utils.py:103-104, :106-110) and the sort of the concatenated scores of
+ * all layers followed by `concatenated_tensor[int(p * len)]` (:139-143, :246-250).  Scores are those of the
+ * pruning calls above (`mode`, `aux`, `aux2`).  A radix select over the scores' bit patterns: three histogram
+ * passes, each over every tensor, and a step after each pass:
+ *     mam_select_begin(ws, bytes, ranks, nranks, stream)         ranks: HOST array of 1 or 2 ascending 0-based ranks
+ *     for pass in 0, 1, 2:
+ *         mam_select_accumulate(ws, w, ldw, mode, aux, aux2, ld_aux, M, K, pass, stream)     once per tensor
+ *         mam_select_advance(ws, pass, stream)
+ *     mam_select_result(ws, mode, out, stream)                   out: DEVICE array of nranks floats
+ * The result is exactly the element a full ascending sort of the |scores| holds at each rank (NaN scores
+ * order above infinity, as torch.sort places them); for MAM_PRUNE_COUNT it is the count as a float.
+ * `ws` is device memory of mam_select_workspace() bytes, 16-byte aligned; nothing synchronises.
+ */
+size_t mam_select_workspace(void);
+int mam_select_begin(void *workspace, size_t workspace_bytes, const int64_t *ranks, int nranks, void *stream);
+int mam_select_accumulate(void *workspace, const float *w, int64_t ldw, int mode, const void *aux,
+                          const void *aux2, int64_t ld_aux, int64_t M, int64_t K, int pass, void *stream);
+int mam_select_advance(void *workspace, int pass, void *stream);
+int mam_select_result(void *workspace, int mode, float *out, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -17,7 +17,7 @@ HIP_LIB = os.path.join(LIB_DIR, "libmam_hip.so")
 OPS_LIB = os.path.join(LIB_DIR, "mam_torch_ops.so")
 
 HIP_SOURCES = ["mam_common.hip", "mam_forward.hip", "mam_backward.hip", "mam_selcount.hip", "mam_csr.hip",
-               "mam_spmm.hip", "mam_prune.hip", "mam_module.hip"]
+               "mam_spmm.hip", "mam_prune.hip", "mam_select.hip", "mam_module.hip"]
 
 # -ffp-contract=off: a product that feeds an add must stay an fp32 multiply followed by an fp32
 # add (bit-exact forward).  Packed-FP32 instructions are disabled for the device pass.

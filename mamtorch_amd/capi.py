@@ -38,6 +38,7 @@ EXPORTS = (
     "mam_csr_spmm", "mam_coo_spmm", "mam_csr_to_dense", "mam_coo_to_dense",
     "mam_blend", "mam_apply_keep", "mam_im2col", "mam_col2im",
     "mam_prune_row_offsets", "mam_prune_fill_csr", "mam_prune_apply",
+    "mam_select_workspace", "mam_select_begin", "mam_select_accumulate", "mam_select_advance", "mam_select_result",
 )
 
 _i64 = ctypes.c_int64
@@ -359,6 +360,36 @@ def prune_to_csr(w, threshold, mode=PRUNE_MAGNITUDE, aux=None, aux2=None):
         _check(l.mam_prune_fill_csr(_p(w), _ld(w), mode, _p(aux), _p(aux2), ld_aux, threshold, _p(crow), _p(col),
                                     _p(val), M, K, _stream(w)))
     return crow, col, val
+
+
+def select_abs_ranks(operands, ranks):
+    """The elements of the given 0-based `ranks` (one or two, ascending) among the absolute scores of all
+    `operands`, each (w, mode, aux, aux2) as for prune_apply (w (M, K) fp32 with contiguous rows): what a
+    full ascending sort of the concatenated |scores| would hold there.  Returns a DEVICE float tensor with
+    one element per rank (reading it is the caller's synchronisation)."""
+    l = lib()
+    l.mam_select_workspace.restype = _size
+    first = operands[0][0]
+    dev = first.device
+    nbytes = l.mam_select_workspace()
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    out = torch.empty(len(ranks), dtype=torch.float32, device=dev)
+    rk = (ctypes.c_int64 * len(ranks))(*[int(r) for r in ranks])
+    mode0 = operands[0][1]
+    with torch.cuda.device(dev):
+        st = _stream(first)
+        _check(l.mam_select_begin(_p(ws), _size(nbytes), rk, len(ranks), st))
+        for ps in range(3):
+            for w, mode, aux, aux2 in operands:
+                if mode != mode0:
+                    raise ValueError("all operands of one selection must use the same score")
+                M, K = w.shape
+                aux, aux2, ld_aux = _prune_operands(w, mode, aux, aux2)
+                _check(l.mam_select_accumulate(_p(ws), _p(w), _i64(_ld(w)), mode, _p(aux), _p(aux2), _i64(ld_aux),
+                                               _i64(M), _i64(K), ps, st))
+            _check(l.mam_select_advance(_p(ws), ps, st))
+        _check(l.mam_select_result(_p(ws), mode0, _p(out), st))
+    return out
 
 
 def prune_apply(w, threshold, mode=PRUNE_MAGNITUDE, aux=None, aux2=None):

@@ -16,28 +16,52 @@ from .. import capi
 
 __all__ = ["layer_threshold", "global_threshold", "prune_", "dense_to_csr"]
 
-_QUANTILE_LIMIT = 16_000_000  # torch.quantile refuses larger inputs
+def _operand(score: Tensor, factor, counts):
+    """(w, mode, aux, aux2) for capi.select_abs_ranks: `score` as a 2-d fp32 matrix with contiguous rows."""
+    t = score.detach()
+    if t.dtype != torch.float32 or t.dim() == 0:
+        t = t.float().reshape(1, -1)
+    if t.dim() != 2 or t.stride(-1) != 1:
+        t = t.reshape(1, -1) if t.is_contiguous() else t.contiguous().reshape(1, -1)
+    mode, aux, aux2 = _mode(t, factor, counts)
+    if aux is not None:
+        aux = aux.reshape(t.shape) if aux.is_contiguous() else aux.contiguous().reshape(t.shape)
+    if aux2 is not None:
+        aux2 = aux2.reshape(t.shape) if aux2.is_contiguous() else aux2.contiguous().reshape(t.shape)
+    return t, mode, aux, aux2
 
 
-def layer_threshold(score: Tensor, p: float) -> float:
-    """``torch.quantile(score.flatten().abs(), p)`` (linear interpolation), also above torch's size limit."""
-    flat = score.detach().flatten().abs().float()
-    if flat.numel() <= _QUANTILE_LIMIT:
-        return float(torch.quantile(flat, p))
-    ordered, _ = torch.sort(flat)
-    pos = p * (flat.numel() - 1)
-    lo = int(pos)
-    hi = min(lo + 1, flat.numel() - 1)
-    a, b = ordered[lo], ordered[hi]
-    return float(a + (b - a) * (pos - lo))
+def layer_threshold(score: Tensor, p: float, factor: Tensor = None, counts=None) -> float:
+    """``torch.quantile(score.flatten().abs(), p)`` (linear interpolation) without sorting and without
+    torch's 16 M element limit: the two neighbours of the quantile are found by a radix select on the device
+    (three histogram passes, capi.select_abs_ranks) and interpolated exactly as torch.quantile does it -- the
+    rank ``p * (n - 1)`` is formed in fp32, its floor and ceiling are the neighbours, ``lerp`` joins them.
+    ``factor`` / ``counts`` choose the score as in :func:`prune_` (weight x factor, selection counts)."""
+    operand = _operand(score, factor, counts)
+    n = operand[0].numel()
+    if n == 0:
+        raise ValueError("no scores")
+    rank = torch.tensor(p, dtype=torch.float32) * (n - 1)
+    lo, hi = int(torch.floor(rank)), int(torch.ceil(rank))
+    lo, hi = max(0, min(lo, n - 1)), max(0, min(hi, n - 1))
+    found = capi.select_abs_ranks([operand], [lo] if hi == lo else [lo, hi]).cpu()
+    below, above = found[0], found[-1]
+    return float(torch.lerp(below, above, rank - torch.floor(rank)))
 
 
-def global_threshold(scores, p: float) -> float:
-    """Element of rank ``int(p * n)`` of the sorted absolute scores of all given tensors."""
-    flat = torch.cat([s.detach().flatten().abs().float() for s in scores])
-    ordered, _ = torch.sort(flat)
-    index = max(0, min(int(p * flat.numel()), flat.numel() - 1))
-    return float(ordered[index])
+def global_threshold(scores, p: float, factors=None, counts=None) -> float:
+    """Element of rank ``int(p * n)`` of the sorted absolute scores of all given tensors, without
+    concatenating or sorting them: every histogram pass of the radix select walks the tensors one by one."""
+    scores = list(scores)
+    factors = [None] * len(scores) if factors is None else list(factors)
+    counts = [None] * len(scores) if counts is None else list(counts)
+    operands = [_operand(s, f, c) for s, f, c in zip(scores, factors, counts)]
+    operands = [o for o in operands if o[0].numel() > 0]
+    n = sum(o[0].numel() for o in operands)
+    if n == 0:
+        raise ValueError("no scores")
+    index = max(0, min(int(p * n), n - 1))
+    return float(capi.select_abs_ranks(operands, [index]).cpu()[0])
 
 
 def _mode(weight, factor, counts):

@@ -131,3 +131,88 @@ def test_full_size_counts_and_order():
     idem = torch.sparse_csr_tensor(crow, col, val, size=(M, K)).to_dense()
     crow2, col2, val2 = capi.prune_to_csr(idem, thr)               # idempotence
     assert torch.equal(crow2, crow) and torch.equal(col2, col) and torch.equal(val2, val)
+
+
+# ---- thresholds by radix select: no sort, bit-equal to the reference's sort-based rules ----
+
+def _sorted_abs(*tensors):
+    return torch.sort(torch.cat([t.detach().abs().float().flatten() for t in tensors]))[0]
+
+
+def _quantile_by_sort(ordered, p):
+    """torch.quantile's linear rule written out (rank formed in fp32, floor / ceil neighbours, lerp), on the
+    CPU: it also covers inputs above torch.quantile's size limit."""
+    n = ordered.numel()
+    rank = torch.tensor(p, dtype=torch.float32) * (n - 1)
+    lo, hi = int(torch.floor(rank)), int(torch.ceil(rank))
+    return float(torch.lerp(ordered[lo].cpu(), ordered[hi].cpu(), rank - torch.floor(rank)))
+
+
+@pytest.mark.parametrize("p", [0.0, 0.5, 0.9, 0.97, 0.999, 1.0])
+def test_layer_threshold_equals_torch_quantile(p):
+    from mamtorch_amd.sparse import prune
+
+    w = (torch.randn(4000, 4000, generator=torch.Generator().manual_seed(2)) * 0.02).to(DEV)   # torch's limit
+    got = prune.layer_threshold(w, p)
+    want = float(torch.quantile(w.flatten().abs().cpu(), p))
+    assert np.float32(got).view(np.int32) == np.float32(want).view(np.int32), (got, want)
+    assert abs(got - float(torch.quantile(w.flatten().abs(), p))) <= 1.2e-7 * abs(want)
+
+
+@pytest.mark.parametrize("p", [0.1, 0.9, 0.99])
+def test_layer_threshold_at_4096_squared(p):
+    """16.8 M scores: above torch.quantile's size limit; the same rule by a full sort is the yardstick."""
+    from mamtorch_amd.sparse import prune
+
+    w = (torch.randn(4096, 4096, generator=torch.Generator().manual_seed(3)) * 0.02).to(DEV)
+    ordered = _sorted_abs(w)
+    got = prune.layer_threshold(w, p)
+    want = _quantile_by_sort(ordered, p)
+    assert np.float32(got).view(np.int32) == np.float32(want).view(np.int32), (got, want)
+
+
+def test_global_threshold_over_three_tensors():
+    """The reference's global rule (sort of the concatenated |scores|, element int(p * n)) over tensors of
+    different shapes, one of them a strided view with an unaligned start."""
+    from mamtorch_amd.sparse import prune
+
+    g = torch.Generator().manual_seed(4)
+    a = (torch.randn(768, 3072, generator=g) * 0.03).to(DEV)
+    b = (torch.randn(3072, 768, generator=g) * 0.01).to(DEV)
+    c = (torch.randn(301, 1031, generator=g)).to(DEV)[:, 3:1001]
+    ordered = _sorted_abs(a, b, c)
+    for p in (0.0, 0.3, 0.9, 0.9999, 1.0):
+        index = max(0, min(int(p * ordered.numel()), ordered.numel() - 1))
+        got = prune.global_threshold([a, b, c], p)
+        assert np.float32(got).view(np.int32) == ordered[index].cpu().numpy().view(np.int32), p
+
+
+def test_thresholds_of_product_and_count_scores_and_corner_cases():
+    from mamtorch_amd.sparse import prune
+
+    g = torch.Generator().manual_seed(5)
+    w = torch.randn(257, 1000, generator=g).to(DEV)
+    grad = torch.randn(257, 1000, generator=g).to(DEV)
+    ordered = _sorted_abs(w * grad)
+    for p in (0.25, 0.9):
+        got = prune.layer_threshold(w, p, factor=grad)
+        assert np.float32(got).view(np.int32) == np.float32(_quantile_by_sort(ordered, p)).view(np.int32)
+        index = int(p * ordered.numel())
+        assert np.float32(prune.global_threshold([w], p, factors=[grad])).view(np.int32) == \
+            ordered[index].cpu().numpy().view(np.int32)
+    cmax = torch.randint(0, 40, (257, 1000), generator=g, dtype=torch.int32).to(DEV)
+    cmin = torch.randint(0, 40, (257, 1000), generator=g, dtype=torch.int32).to(DEV)
+    ordered = torch.sort((cmax + cmin).flatten().float())[0]
+    for p in (0.1, 0.5, 0.95):
+        assert prune.global_threshold([w], p, counts=[(cmax, cmin)]) == float(ordered[int(p * ordered.numel())])
+    # ties, signed zeros, a single element, NaN scores (they order above infinity, where torch.sort puts them)
+    t = torch.tensor([[0.0, -0.0, 1.0, -1.0, 1.0, float("inf"), float("nan"), -2.0]], device=DEV)
+    ordered = torch.sort(t.abs().flatten())[0]
+    for index in range(8):
+        got = prune.global_threshold([t], (index + 0.5) / 8)
+        want = float(ordered[index])
+        assert (got != got and want != want) or got == want, (index, got, want)
+    assert prune.global_threshold([torch.tensor([[-3.5]], device=DEV)], 0.7) == 3.5
+    assert prune.layer_threshold(torch.tensor([[-3.5]], device=DEV), 0.7) == 3.5
+    same = torch.full((64, 64), -0.25, device=DEV)
+    assert prune.layer_threshold(same, 0.33) == 0.25 and prune.global_threshold([same, same], 0.99) == 0.25
