@@ -48,7 +48,7 @@ extern "C" {
                                  likewise for min (the retired convolution modules' literal rule)        */
 
 /* Run-time switches for mam_set_option().  Their initial values come from the environment variables of
- * the same names, read once when the library is loaded: MAM_FORWARD_TILING = auto | wide | 0 | 1 | 2,
+ * the same names, read once when the library is loaded: MAM_FORWARD_TILING = auto | wide | 0 | 1 | 2 | 3,
  * MAM_BACKWARD_FORK = auto | -1 | 0 | 1, MAM_BACKWARD_ONE_LAUNCH = auto | 0 (off) | 1 (auto) | 2 (on),
  * MAM_BACKWARD_EXACT = 0 | 1.  A value outside an
  * option's range is refused by mam_set_option() and ignored (with the default kept) in the environment. */
@@ -60,6 +60,8 @@ extern "C" {
 #define MAM_FORWARD_TILING_AUTO 0 /* wave-uniform-rows tiling where the layout allows it           */
 #define MAM_FORWARD_TILING_WIDE 1 /* every call on the general 64 x 128 tiling                     */
 #define MAM_FORWARD_TILING_GROUPS16 2 /* as AUTO, but indices recorded per 16 products at every K   */
+#define MAM_FORWARD_TILING_FUSED_MERGE 3 /* as AUTO, but a K-split call merges inside the forward launch: the
+                                            last of a tile's workgroups to finish combines and resolves   */
 #define MAM_BACKWARD_FORK_AUTO (-1) /* from 2^22 outputs on, and under stream capture from 2^16   */
 #define MAM_BACKWARD_FORK_OFF 0
 #define MAM_BACKWARD_FORK_ON 1
@@ -142,7 +144,9 @@ int mam_fc_forward_describe(const float *x, int64_t ldx, const float *w, int64_t
  * mam_fc_forward_static_limit() guarantees a fit; the query covers the worst alignment, so a call may fit
  * although it says more).  It calls no allocating routine.  All calls on one GPU share that GPU's
  * array: calls that may overlap on one GPU (different streams, different threads) race on it -- serialise
- * them, or use mam_fc_forward with one workspace per stream.  Nothing in the array has to be cleared
+ * them, or use mam_fc_forward with one workspace per stream.  The first call on a device performs that
+ * device's one-time set-up (kernel attributes, the array's address; the library's second stream is left for
+ * the first call outside a capture) unless mam_init() ran there before.  Nothing in the array has to be cleared
  * between calls (a call writes every word it later reads).
  */
 size_t mam_fc_forward_static_limit(void);
@@ -168,6 +172,14 @@ int mam_fc_forward_values(const float *x, int64_t ldx, const float *w, int64_t l
  * Either output pointer may be NULL to skip it.  grad/argmax/argmin are (N,M) contiguous.
  * `w_sel` and `x_sel` (optional, each may be NULL) are the (2, N, M) arrays written by mam_fc_forward for
  * the same inputs; x_grad uses w_sel, w_grad uses x_sel, and whichever is NULL is gathered from w / x.
+ * Summation: each term is one fp32 product.  x_grad is accumulated in 64-bit fixed-point cells and is the
+ * exact sum of its terms rounded once (independent of the order of arrival, the same bits on every call) as
+ * long as at most 512 terms of one workgroup's slab (a batch row, or a few of them) fall outside a window
+ * that reaches ~2^25 below the slab's largest term; such terms are added in fp64 before the one rounding,
+ * and a slab with more of them is summed with fp32 atomics instead (order-dependent, within rtol 1e-5 plus
+ * the rounding floor of an fp32 sum).  w_grad is summed in fp32 in no fixed order, as the reference's
+ * atomicAdd does, unless MAM_OPT_BACKWARD_EXACT is on: then it is accumulated the same exact way ((M,K)
+ * weights, 16-byte aligned operands, M and K multiples of 4; other calls keep the fp32 route).
  * Replaces fullyconnected_backward_cuda
  * (mamtorch/kernel/v4/csrc/cuda/fullyconnected_backward.cu:80-135, kernel :24-78; v1 identical).
  * Indices outside [0,K) make the call's result undefined for that output only (they are skipped).

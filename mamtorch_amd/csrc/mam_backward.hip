@@ -18,8 +18,11 @@
 //            by several workgroups per slab, which add their shares to the cleared w_grad.
 //
 // Each term is one fp32 product (operand of the reference's atomicAdd).  x_grad is the exact sum of its
-// terms rounded once; in w_grad only the order of the fp32 additions differs from the reference, which is
-// itself unordered.
+// terms rounded once -- as long as at most QCAP (512) terms of a workgroup's slab fall outside its
+// fixed-point window (they are added in fp64 before the rounding); a slab with more of them falls back to
+// fp32 LDS atomics and is then a sum in arrival order.  In w_grad only the order of the fp32 additions
+// differs from the reference, which is itself unordered; option MAM_OPT_BACKWARD_EXACT accumulates it in
+// fixed-point cells as well (mam_bwd_w_exact_kernel).
 #include "mam_common.h"
 #include "mam_fixed.h"
 #include "mam_count_stream.h"

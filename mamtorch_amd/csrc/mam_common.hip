@@ -120,7 +120,7 @@ int g_num_hooks = 0;
 // The values each option accepts.
 struct OptionRange { const char *env; int lo, hi, fallback; bool wide_word; };
 constexpr OptionRange kOptionRanges[MAM_OPT_COUNT_] = {
-    {"MAM_FORWARD_TILING", MAM_FORWARD_TILING_AUTO, MAM_FORWARD_TILING_GROUPS16, MAM_FORWARD_TILING_AUTO, true},
+    {"MAM_FORWARD_TILING", MAM_FORWARD_TILING_AUTO, MAM_FORWARD_TILING_FUSED_MERGE, MAM_FORWARD_TILING_AUTO, true},
     {"MAM_BACKWARD_FORK", MAM_BACKWARD_FORK_AUTO, MAM_BACKWARD_FORK_ON, MAM_BACKWARD_FORK_AUTO, false},
     {"MAM_BACKWARD_ONE_LAUNCH", MAM_BACKWARD_ONE_LAUNCH_OFF, MAM_BACKWARD_ONE_LAUNCH_ON, MAM_BACKWARD_ONE_LAUNCH_AUTO,
      false},

@@ -476,3 +476,36 @@ def test_nan_products_are_ignored():
         x[6, 17] = float("nan")
         w[6, 17] = float("nan")
         _run_both_layouts(x, w, None, "nan products %dx%dx%d" % (N, K, M))
+
+
+def test_merge_inside_the_forward_launch_gives_the_same_bits():
+    """MAM_FORWARD_TILING_FUSED_MERGE: the last of a tile's workgroups to finish combines the K ranges and resolves
+    in its own epilogue (no merge kernel).  Kept for comparisons (it is slower: 0.234 against 0.212 ms at
+    256 x 4096 x 4096); its results must be those of the shipped pair, and of the oracle."""
+    from mamtorch_amd import capi
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(31)
+    for N, K, M in ((48, 2048, 256), (100, 4096, 200)):
+        x = torch.randn(N, K, generator=g)
+        w = torch.randn(M, K, generator=g)
+        x[3, :] = 0.0                       # ties and zero signs across the K ranges
+        w[5, K // 2:] = w[5, :K // 2]
+        want = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+        xd, wd = x.to(dev), w.to(dev)
+        ws = torch.empty(2, N, M, device=dev)
+        xs = torch.empty(2, N, M, device=dev)
+        capi.set_option(capi.OPT_FORWARD_TILING, 3)
+        try:
+            assert "split" in capi.fc_forward_describe(xd, wd, capi.W_MK)
+            for _ in range(2):              # the tickets are cleared per call
+                c, amax, amin = capi.fc_forward(xd, wd, capi.W_MK, w_sel=ws, x_sel=xs)
+                torch.cuda.synchronize()
+                assert_bits_equal(c.cpu().numpy(), want[0], "fused merge c")
+                assert_index_equal(amax.cpu().numpy(), want[1], "fused merge argmax")
+                assert_index_equal(amin.cpu().numpy(), want[2], "fused merge argmin")
+        finally:
+            capi.set_option(capi.OPT_FORWARD_TILING, capi.FORWARD_TILING_AUTO)
+        cols = torch.arange(M)[None, :]
+        assert torch.equal(ws[0].cpu(), w[cols, torch.tensor(want[1]).long()])
+        assert torch.equal(xs[1].cpu(), x[torch.arange(N)[:, None], torch.tensor(want[2]).long()])
