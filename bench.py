@@ -761,12 +761,12 @@ def run_module(torch, capi, lib, dev, args):
                             "by_phase_ms": {k: round(ph[k] - ph_cabi[k], 5) for k in ph},
                             "what": "per step: at::empty of c, argmax, argmin, the (4,N,M) hand-over tensor and the "
                                     "split-K workspace in the forward; at::empty of both gradients, the bias "
-                                    "gradient (a column sum by ATen) and autograd's bookkeeping in the backward"},
+                                    "gradient (mam_bias_grad, one more kernel) and autograd's bookkeeping in the backward"},
         "roofline": valu_roofline("; ".join(sorted(set(L.describe() for L in cl))) + " behind the module",
                                   triples, ph["forward"]),
         "fwd_bwd_gops": round(triples / ((ph["forward"] + ph["backward"]) * 1e-3) / 1e9, 2),
         "fwd_bwd_valu_frac": round(3.0 * triples / ((ph["forward"] + ph["backward"]) * 1e-3) / 1e12 / VALU_PEAK_TFLOPS, 4),
-        "roofline_backward": hbm_roofline("mam_bwd_x_kernel + mam_bwd_w_vec_kernel behind autograd (+ bias column sum)",
+        "roofline_backward": hbm_roofline("mam_bwd_x_kernel + mam_bwd_w_vec_kernel + col_sum_kernel behind autograd",
                                           bwd_bytes, ph["backward"]),
     }
     cpu = None

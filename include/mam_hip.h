@@ -314,6 +314,16 @@ int mam_blend(const float *mam_out, const float *mac_out, const float *bias, flo
               int64_t N, int64_t M, void *stream);
 
 /*
+ * bias_grad[m] = sum over the batch rows of grad[n, m]: the gradient of the bias the layer adds after max + min
+ * (mamtorch/nn/v4/fullyconnected.py:197-198; in the reference autograd derives this column sum from the `+`).
+ * fp32 adds in a fixed order (the same bits on every call).  `workspace`: mam_bias_grad_workspace(N, M) bytes
+ * (0 up to 512 batch rows).
+ */
+size_t mam_bias_grad_workspace(int64_t N, int64_t M);
+int mam_bias_grad(const float *grad, int64_t ld, float *bias_grad, int64_t N, int64_t M, void *workspace,
+                  size_t workspace_bytes, void *stream);
+
+/*
  * out (M, K) contiguous = w (M, K, row stride ldw) * (keep ? 1 : 0), keep (M, K) contiguous bytes: the
  * training-time weight dropout of the module (mamtorch/nn/v4/fullyconnected.py:143-148, there a float
  * Bernoulli mask of the weight's size times the transposed weight) in one pass from a byte mask.  The

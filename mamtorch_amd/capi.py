@@ -36,7 +36,7 @@ EXPORTS = (
     "mam_fc_forward_ranges_workspace", "mam_fc_forward_ranges", "mam_fc_backward_ranges",
     "mam_csr_fc_forward_workspace", "mam_csr_fc_forward", "mam_csr_fc_backward", "mam_csr_validate",
     "mam_csr_spmm", "mam_coo_spmm", "mam_csr_to_dense", "mam_coo_to_dense",
-    "mam_blend", "mam_apply_keep", "mam_im2col", "mam_col2im",
+    "mam_blend", "mam_bias_grad_workspace", "mam_bias_grad", "mam_apply_keep", "mam_im2col", "mam_col2im",
     "mam_prune_row_offsets", "mam_prune_fill_csr", "mam_prune_apply",
     "mam_select_workspace", "mam_select_begin", "mam_select_accumulate", "mam_select_advance", "mam_select_result",
 )

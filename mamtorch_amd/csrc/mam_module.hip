@@ -188,7 +188,93 @@ static int make_geom(ConvGeom &g, int64_t B, int64_t C, int64_t H, int64_t W, in
 }
 
 }  // namespace module
+// Column sums of grad (N, M): the gradient of the bias that the layer adds after max + min
+// (mamtorch/nn/v4/fullyconnected.py:197-198; the reference leaves this sum to autograd).  A workgroup owns 64
+// columns and a slab of the batch rows: its four waves take every fourth row of the slab (a row piece of 64
+// columns is one coalesced 256-byte load, eight of them in flight per wave), add in row order, and the four
+// partial sums are added in wave order -- the result does not depend on timing.  With several slabs the
+// partial rows go to the workspace and a second launch adds them in slab order.
+__global__ __launch_bounds__(256) void col_sum_kernel(const float *__restrict__ grad, int64_t ld,
+                                                      float *__restrict__ out, int N, int M, int rows_per_slab)
+{
+    __shared__ float part[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = blockIdx.x * 64 + lane;
+    const int n_begin = blockIdx.y * rows_per_slab;
+    const int n_end = (n_begin + rows_per_slab) < N ? (n_begin + rows_per_slab) : N;
+    float acc = 0.0f;
+    if (m < M) {
+        const float *col = grad + m;
+        int n = n_begin + wave;
+        for (; n + 28 < n_end; n += 32) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = col[(int64_t)(n + 4 * u) * ld];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += v[u];
+        }
+        for (; n < n_end; n += 4) acc += col[(int64_t)n * ld];
+    }
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && m < M)
+        out[(int64_t)blockIdx.y * M + m] = ((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane];
+}
+
+__global__ __launch_bounds__(256) void slab_sum_kernel(const float *__restrict__ partial, float *__restrict__ out,
+                                                       int M, int slabs)
+{
+    const int m = blockIdx.x * 256 + threadIdx.x;
+    if (m >= M) return;
+    float acc = 0.0f;
+    for (int s = 0; s < slabs; ++s) acc += partial[(int64_t)s * M + m];
+    out[m] = acc;
+}
+
+// slabs of the batch: one up to 512 rows, else slabs of at least 128 rows, at most 64 of them
+static int64_t bias_grad_slabs(int64_t N)
+{
+    if (N <= 512) return 1;
+    int64_t s = N / 128;
+    return s > 64 ? 64 : s;
+}
+
 }  // namespace mam
+
+extern "C" size_t mam_bias_grad_workspace(int64_t N, int64_t M)
+{
+    if (N <= 0 || M <= 0) return 0;
+    const int64_t slabs = mam::bias_grad_slabs(N);
+    return slabs > 1 ? (size_t)slabs * (size_t)M * sizeof(float) : 0;
+}
+
+extern "C" int mam_bias_grad(const float *grad, int64_t ld, float *bias_grad, int64_t N, int64_t M, void *workspace,
+                             size_t workspace_bytes, void *stream)
+{
+    using namespace mam;
+    if (N < 0 || M < 0) return fail(MAM_ERR_INVALID_ARGUMENT, "negative size");
+    if (M == 0) return MAM_OK;
+    if (!bias_grad) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (N == 0) return fill_zero(bias_grad, M, st);
+    if (!grad) return fail(MAM_ERR_INVALID_ARGUMENT, "null pointer");
+    if (ld < M) return fail(MAM_ERR_INVALID_ARGUMENT, "ld smaller than the number of columns");
+    if (N > INT32_MAX / 2 || M > INT32_MAX / 2) return fail(MAM_ERR_UNSUPPORTED, "a dimension exceeds 2^30");
+    const int64_t slabs = bias_grad_slabs(N);
+    const size_t need = slabs > 1 ? (size_t)slabs * (size_t)M * sizeof(float) : 0;
+    if (need > 0 && (!workspace || workspace_bytes < need))
+        return fail(MAM_ERR_WORKSPACE, "the bias gradient needs %zu workspace bytes, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    const int64_t rows_per_slab = ceil_div(N, slabs);
+    float *first = slabs > 1 ? static_cast<float *>(workspace) : bias_grad;
+    hipLaunchKernelGGL(col_sum_kernel, dim3((unsigned)ceil_div(M, 64), (unsigned)slabs), dim3(256), 0, st, grad, ld, first,
+                       (int)N, (int)M, (int)rows_per_slab);
+    int rc = check_launch("col_sum_kernel");
+    if (rc != MAM_OK || slabs == 1) return rc;
+    hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)ceil_div(M, 256)), dim3(256), 0, st, first, bias_grad, (int)M,
+                       (int)slabs);
+    return check_launch("slab_sum_kernel");
+}
 
 extern "C" int mam_blend(const float *mam_out, const float *mac_out, const float *bias, float alpha, float beta,
                          float *out, int64_t N, int64_t M, void *stream)

@@ -307,6 +307,22 @@ at::Tensor blend(const at::Tensor &mam, const at::Tensor &mac, const c10::option
     return out;
 }
 
+// column sums of the output gradient: the bias gradient of the layer
+at::Tensor bias_grad(const at::Tensor &grad)
+{
+    check_f32_2d(grad, "grad");
+    const int64_t N = grad.size(0), M = grad.size(1);
+    const c10::DeviceGuard guard(grad.device());
+    const at::Tensor g = grad.stride(1) == 1 ? grad : grad.contiguous();
+    auto out = at::empty({M}, grad.options());
+    const size_t ws_bytes = mam_bias_grad_workspace(N, M);
+    auto ws = workspace_for(ws_bytes, grad);
+    check_rc(mam_bias_grad(g.data_ptr<float>(), g.stride(0), out.data_ptr<float>(), N, M,
+                           ws.defined() ? ws.data_ptr() : nullptr, ws_bytes, current_stream(grad)),
+             "mam_bias_grad");
+    return out;
+}
+
 // weight (out, in) times a {0, 1} mask kept as bool / uint8: the module's weight dropout and its gradient
 at::Tensor apply_keep(const at::Tensor &w, const at::Tensor &keep)
 {
@@ -550,6 +566,7 @@ TORCH_LIBRARY(mamtorch_kernel_v4, m)
     m.def("fullyconnected_ranges(Tensor a, Tensor weight, Tensor? bias, int range_len, bool with_indices) -> Tensor[]");
     m.def("fullyconnected_ranges_backward(Tensor a, Tensor weight, Tensor grad, Tensor argmax, Tensor argmin, int range_len) -> Tensor[]");
     m.def("blend(Tensor mam, Tensor mac, Tensor? bias, float alpha, float beta) -> Tensor");
+    m.def("bias_grad(Tensor grad) -> Tensor");
     m.def("apply_keep(Tensor weight, Tensor keep) -> Tensor");
     m.def("im2col(Tensor x, int k1, int k2, int s1, int s2) -> Tensor");
     m.def("col2im(Tensor cols, int B, int C, int H, int W, int k1, int k2, int s1, int s2) -> Tensor");
@@ -583,6 +600,7 @@ TORCH_LIBRARY_IMPL(mamtorch_kernel_v4, CUDA, m)
     m.impl("fullyconnected_ranges", &fullyconnected_ranges);
     m.impl("fullyconnected_ranges_backward", &fullyconnected_ranges_backward);
     m.impl("blend", &blend);
+    m.impl("bias_grad", &bias_grad);
     m.impl("apply_keep", &apply_keep);
     m.impl("im2col", &im2col);
     m.impl("col2im", &col2im);

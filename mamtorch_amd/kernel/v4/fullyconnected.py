@@ -83,7 +83,7 @@ def _wt_backward(ctx, grad):
     if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
         a_grad, w_grad = K.fullyconnected_wt_backward.default(a, weight, g.contiguous(), argmax, argmin, sel)
     if ctx.needs_input_grad[2]:
-        bias_grad = g.sum(dim=0)
+        bias_grad = K.bias_grad.default(g)
     return a_grad, w_grad, bias_grad, None
 
 

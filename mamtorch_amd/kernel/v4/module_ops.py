@@ -58,7 +58,7 @@ def _ranges_backward(ctx, grad):
         a_grad, w_grad = K.fullyconnected_ranges_backward.default(a, weight, g.contiguous(), argmax, argmin,
                                                                   ctx.range_len)
     if ctx.needs_input_grad[2]:
-        bias_grad = g.sum(dim=0)
+        bias_grad = K.bias_grad.default(g)
     return a_grad, w_grad, bias_grad, None, None
 
 
@@ -87,6 +87,12 @@ def col2im(cols: Tensor, shape, k1: int, k2: int, s1: int, s2: int) -> Tensor:
     """Adjoint of :func:`im2col`: (B * L1 * L2, k2 * k1 * C) -> (B, C, H, W), overlapping windows add up."""
     B, C, H, W = shape
     return K.col2im.default(cols, B, C, H, W, k1, k2, s1, s2)
+
+
+@torch.library.register_fake("mamtorch_kernel_v4::bias_grad")
+def _(grad):
+    torch._check(grad.dim() == 2 and grad.dtype == torch.float)
+    return torch.empty((grad.size(1),), dtype=torch.float, device=grad.device)
 
 
 @torch.library.register_fake("mamtorch_kernel_v4::blend")

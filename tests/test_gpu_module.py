@@ -345,3 +345,29 @@ def test_legacy_layers_against_the_oracle():
         c_mam = oracle.forward(x.reshape(-1, 40).numpy(), w.numpy(), oracle.W_MK)[0]
         want = (0.75 * torch.from_numpy(c_mam) + b.view(1, -1)).view(5, 7, 24) + 0.25 * torch.nn.functional.linear(x, w)
         assert torch.allclose(y2, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("N,M", [(1, 1), (64, 256), (256, 4096), (513, 70), (1300, 333), (12608, 768)])
+def test_bias_gradient_is_the_column_sum(N, M):
+    """The layer's bias gradient (autograd of the `+ bias` after max + min, mamtorch/nn/v4/fullyconnected.py:197-198)
+    as one kernel: column sums in a fixed order, the same bits on every call, against the fp64 sum."""
+    g = torch.randn(N, M, generator=torch.Generator().manual_seed(N + M)).to(DEV)
+    got = torch.ops.mamtorch_kernel_v4.bias_grad(g)
+    again = torch.ops.mamtorch_kernel_v4.bias_grad(g)
+    want = g.double().sum(dim=0)
+    floor = g.abs().double().sum(dim=0)
+    assert got.shape == (M,) and torch.equal(got, again)
+    assert bool(((got.double() - want).abs() <= 1e-5 * want.abs() + 2.0 ** -22 * floor).all())
+    # a strided view (every other column block of a wider matrix)
+    wide = torch.randn(N, 2 * M + 3, generator=torch.Generator().manual_seed(7)).to(DEV)
+    view = wide[:, 3:3 + M]
+    assert bool(((torch.ops.mamtorch_kernel_v4.bias_grad(view).double() - view.double().sum(dim=0)).abs()
+                 <= 1e-5 * view.double().sum(dim=0).abs() + 2.0 ** -22 * view.abs().double().sum(dim=0)).all())
+
+
+def test_bias_gradient_through_the_module():
+    layer = mt.nn.FullyConnected(96, 40, bias=True).to(DEV).train()
+    x = torch.randn(50, 96, generator=torch.Generator().manual_seed(3)).to(DEV).requires_grad_(True)
+    g = torch.randn(50, 40, generator=torch.Generator().manual_seed(4)).to(DEV)
+    layer(x).backward(g)
+    torch.testing.assert_close(layer.bias.grad, g.sum(dim=0), rtol=1e-5, atol=1e-5)
