@@ -70,6 +70,7 @@ struct Params {
     int vec_x, vec_w;  // 16-byte global loads are legal for x / w
     int fast;          // the k-invariant 32-bit-offset staging path is legal
     int coop;          // the cooperative resolve is legal: (M,K) w, 16-byte rows, K % G == 0
+    int group_n;       // row tiles swept under one W panel (tile order of the launch)
     int gt;            // products per recorded group: G, or 2 G on the wave-uniform-rows tiling at large K
 };
 
@@ -486,10 +487,10 @@ __global__ __launch_bounds__(NT, 2) void mam_fwd_kernel(const Params p)
     const int tiles = p.tiles_n * p.tiles_m;
     const int split = logical / tiles;
     const int l = logical - split * tiles;
-    const int per_group = GROUP_N * p.tiles_m;
+    const int per_group = p.group_n * p.tiles_m;
     const int grp = l / per_group;
-    const int first_n = grp * GROUP_N;
-    const int gsize = (p.tiles_n - first_n) < GROUP_N ? (p.tiles_n - first_n) : GROUP_N;
+    const int first_n = grp * p.group_n;
+    const int gsize = (p.tiles_n - first_n) < p.group_n ? (p.tiles_n - first_n) : p.group_n;
     const int lin = l - grp * per_group;
     const int tn = first_n + lin % gsize;
     const int tm = lin / gsize;
@@ -882,10 +883,10 @@ __global__ __launch_bounds__(sx::NT, 4) void mam_fwd_sx_kernel(const Params p)
     const int tiles = p.tiles_n * p.tiles_m;
     const int split = logical / tiles;
     const int l = logical - split * tiles;
-    const int per_group = GROUP_N * p.tiles_m;
+    const int per_group = p.group_n * p.tiles_m;
     const int grp = l / per_group;
-    const int first_n = grp * GROUP_N;
-    const int gsize = (p.tiles_n - first_n) < GROUP_N ? (p.tiles_n - first_n) : GROUP_N;
+    const int first_n = grp * p.group_n;
+    const int gsize = (p.tiles_n - first_n) < p.group_n ? (p.tiles_n - first_n) : p.group_n;
     const int lin = l - grp * per_group;
     const int tn = first_n + lin % gsize;
     const int tm = lin / gsize;
@@ -1280,6 +1281,12 @@ static int make_plan(Plan &plan, bool args, const float *x, int64_t ldx, const f
     const int bn = use_sx ? sx::BN : BN, bm = use_sx ? sx::BM_MAX : BM;
     p.tiles_n = (int)ceil_div(N, bn);
     p.tiles_m = (int)ceil_div(M, bm);
+    // Tile order: GROUP_N row tiles are swept under one W panel, panel after panel.  An XCD has 64 tiles in
+    // flight; with fewer than 8 panels a group of 8 row tiles is shorter than that and the window straddles
+    // groups, every panel of W in flight at once.  Groups of 64 row tiles keep one panel at a time there
+    // (12608 x 3072 -> 768, 6 panels: 1.585 -> 1.517 ms; with 8 or more panels groups of 16 to 128 row tiles
+    // change nothing or lose: 16384 x 4096 -> 1024 3.13 -> 3.29 ms at 64).
+    p.group_n = p.tiles_m < 8 ? 8 * GROUP_N : GROUP_N;
     if (range_len > 0) {
         p.k_per_split = (int)(range_len < K ? range_len : K);
     } else {
