@@ -55,8 +55,8 @@ HBM_PEAK_GBS = 8000.0
 # what the same counter reads for the plain 64 MiB copy made before the warm-up); they are not measured
 # by the run that prints them.
 TRAFFIC_PROFILE = "profiles/hbm_traffic_headline_n256_k4096_m4096.md"
-FORWARD_TRAFFIC_BYTES = {"mam_fwd_sx_kernel": 135.9e6, "mam_fwd_merge_kernel": 141.6e6}
-BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.3e6, "mam_bwd_w_vec_kernel": 90.9e6}
+FORWARD_TRAFFIC_BYTES = {"mam_fwd_sx_kernel": 136.2e6, "mam_fwd_merge_kernel": 141.4e6}
+BACKWARD_TRAFFIC_BYTES = {"mam_bwd_x_kernel": 25.3e6, "mam_bwd_w_vec_kernel": 91.1e6}
 SELCOUNT_TRAFFIC_BYTES = {"selcount_kernel": 166.4e6}
 RAMP_MIN_CALLS = 300          # untimed phase calls before the counted warm-up: the GPU clock ramps over them
 RAMP_MIN_SECONDS = 0.3
@@ -537,7 +537,7 @@ def run_spmm_sweep(torch, capi, lib, dev, args):
                 asp = ad.to_sparse(layout=layout)
                 ms = timed(lambda: op(asp, b), steps)
                 lib_ms = timed(lambda: torch.sparse.mm(asp, b), max(steps // 4, 3))
-                dense_route = size >= 64 and nnz * 8 >= size * size
+                dense_route = size >= 64 and nnz * (16 if name == "coo" else 8) >= size * size
                 cells.append({"size": size, "sparse_rate": rate, "layout": name, "nnz": nnz,
                               "cusparsemm_ms": round(ms, 5), "torch_matmul_dense_ms": round(dense_ms, 5),
                               "torch_sparse_mm_ms": round(lib_ms, 5),

@@ -490,9 +490,12 @@ void check_spmm_operands(const at::Tensor &a, const at::Tensor &b)
 // dense fp32 GEMM over the zero-filled operand: the operand is written out dense (one pass) and the
 // product is the platform's library GEMM.  4096 x 4096 x 4096: 3.06 -> ~1.05 ms at 30 % density; the two
 // routes cross at ~10 %.
-bool dense_route_pays(int64_t nnz, int64_t R, int64_t K, int64_t C)
+// `one_in`: the density from which the route is taken, one stored entry in `one_in`: 8 for CSR; 16 for COO,
+// whose kernel (any order, duplicates, atomics) takes about twice the CSR kernel's time per entry (4096^3 at
+// 10 % density: 1.89 against 1.05 ms, the GEMM 0.99 ms).
+bool dense_route_pays(int64_t nnz, int64_t R, int64_t K, int64_t C, int64_t one_in)
 {
-    return R > 0 && K > 0 && C >= 64 && nnz >= (R * K + 7) / 8 && R * K <= (int64_t(1) << 29);
+    return R > 0 && K > 0 && C >= 64 && nnz >= (R * K + one_in - 1) / one_in && R * K <= (int64_t(1) << 29);
 }
 
 at::Tensor cusparsemm_csr(const at::Tensor &a, const at::Tensor &b)
@@ -504,7 +507,7 @@ at::Tensor cusparsemm_csr(const at::Tensor &a, const at::Tensor &b)
     const at::Tensor crow = a.crow_indices().to(at::kLong).contiguous();
     const at::Tensor col = a.col_indices().to(at::kLong).contiguous();
     const at::Tensor val = a.values().contiguous();
-    if (dense_route_pays(val.numel(), R, K, C)) {
+    if (dense_route_pays(val.numel(), R, K, C, 8)) {
         auto dense = at::empty({R, K}, b.options());
         check_rc(mam_csr_to_dense(crow.data_ptr<int64_t>(), col.data_ptr<int64_t>(), val.data_ptr<float>(),
                                   dense.data_ptr<float>(), K, R, K, current_stream(b)),
@@ -530,7 +533,7 @@ at::Tensor cusparsemm_coo(const at::Tensor &a, const at::Tensor &b)
     const at::Tensor idx = a._indices().to(at::kLong).contiguous();   // (2, nnz); need not be coalesced
     const at::Tensor val = a._values().contiguous();
     const int64_t nnz = val.numel();
-    if (dense_route_pays(nnz, R, K, C)) {
+    if (dense_route_pays(nnz, R, K, C, 16)) {
         auto dense = at::empty({R, K}, b.options());
         check_rc(mam_coo_to_dense(idx.data_ptr<int64_t>(), idx.data_ptr<int64_t>() + nnz, val.data_ptr<float>(), nnz,
                                   dense.data_ptr<float>(), K, R, K, current_stream(b)),

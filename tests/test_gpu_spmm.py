@@ -152,11 +152,11 @@ def test_operator_at_high_density(layout, n, l, m, rate):
 @pytest.mark.parametrize("layout", [torch.sparse_csr, torch.sparse_coo])
 @pytest.mark.parametrize("above", [False, True])
 def test_operator_either_side_of_the_density_threshold(layout, above):
-    """The operator changes route at one stored entry in eight (sparse kernel below, dense copy + library GEMM
-    from there on), and with it the order of summation: one entry below and exactly at the threshold, both
-    against the fp64 defining sum within rtol 1e-5 plus the rounding floor of an fp32 sum."""
+    """The operator changes route at one stored entry in eight (CSR; one in sixteen for COO): sparse kernel below,
+    dense copy + library GEMM from there on, and with it the order of summation: one entry below and exactly at
+    the threshold, both against the fp64 defining sum within rtol 1e-5 plus the rounding floor of an fp32 sum."""
     R, K, C = 96, 256, 128
-    nnz = R * K // 8 + (0 if above else -1)
+    nnz = R * K // (8 if layout == torch.sparse_csr else 16) + (0 if above else -1)
     g = torch.Generator().manual_seed(17 + int(above))
     where = torch.randperm(R * K, generator=g)[:nnz]
     a = torch.zeros(R * K)
