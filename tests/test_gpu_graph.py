@@ -128,3 +128,74 @@ def test_sparse_step_replays():
         mask = (dense != 0).numpy()
         _close(vg, wo[mask], wa[mask], tag + " val_grad")
         torch.randn(128, 128, device=dev).sum().item()
+
+
+def test_backward_count_exact_option_and_select_replay():
+    """The one-call backward + selection count (fused kernel), the backward with MAM_OPT_BACKWARD_EXACT and the
+    radix select of a threshold, recorded once and replayed on changing inputs: counts exact, the exact option's
+    gradients bit-equal to the fp64-accumulated oracle, the selected element equal to the sorted one."""
+    from mamtorch_amd import capi
+
+    dev = torch.device("cuda:0")
+    N, K, M = 128, 2048, 256
+    cases = [random_case(N, K, M, seed=40 + s) for s in range(3)]
+    xs = torch.empty(N, K, device=dev)
+    ws = torch.empty(M, K, device=dev)
+    gs = torch.empty(N, M, device=dev)
+    w_sel = torch.empty(2, N, M, device=dev)
+    x_sel = torch.empty(2, N, M, device=dev)
+    max_count = torch.zeros(M, K, dtype=torch.int32, device=dev)
+    min_count = torch.zeros(M, K, dtype=torch.int32, device=dev)
+    rank = (M * K * 9) // 10
+
+    def step():
+        c, amax, amin = capi.fc_forward(xs, ws, capi.W_MK, w_sel=w_sel, x_sel=x_sel)
+        xg, wg = capi.fc_backward_count(xs, ws, gs, amax, amin, max_count, min_count, capi.COUNT_HITS, capi.W_MK,
+                                        w_sel=w_sel, x_sel=x_sel)
+        capi.set_option(capi.OPT_BACKWARD_EXACT, 1)
+        try:
+            xe, we = capi.fc_backward(xs, ws, gs, amax, amin, capi.W_MK, w_sel=w_sel, x_sel=x_sel)
+        finally:
+            capi.set_option(capi.OPT_BACKWARD_EXACT, 0)
+        found = capi.select_abs_ranks([(ws, capi.PRUNE_MAGNITUDE, None, None)], [rank])
+        return amax, amin, xg, wg, xe, we, found
+
+    def load(case):
+        x, w, g = case
+        xs.copy_(x)
+        ws.copy_(w)
+        gs.copy_(g)
+
+    load(cases[0])
+    step()
+    torch.cuda.synchronize()
+    max_count.zero_()
+    min_count.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step()
+    want_max = np.zeros((M, K), np.int64)
+    want_min = np.zeros((M, K), np.int64)
+    for r, case in enumerate(cases + cases[:1]):
+        load(case)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        amax, amin, xg, wg, xe, we, found = (t.cpu().numpy() for t in outs)
+        x, w, g = case
+        want = oracle.forward(x.numpy(), w.numpy(), oracle.W_MK)
+        tag = "replay %d" % r
+        assert_index_equal(amax, want[1], tag + " argmax")
+        assert_index_equal(amin, want[2], tag + " argmin")
+        xo, wo = oracle.backward(x.numpy(), w.numpy(), g.numpy(), want[1], want[2], oracle.W_MK)
+        xa, wa = oracle.backward(x.abs().numpy(), w.abs().numpy(), g.abs().numpy(), want[1], want[2], oracle.W_MK)
+        _close(xg, xo, xa, tag + " x_grad (one call with the count)")
+        _close(wg, wo, wa, tag + " w_grad (one call with the count)")
+        assert_bits_equal(xe, xo.astype(np.float32), tag + " x_grad (exact option)")
+        assert_bits_equal(we, wo.astype(np.float32), tag + " w_grad (exact option)")
+        np.add.at(want_max, (np.arange(M)[None, :].repeat(N, 0), want[1]), 1)
+        np.add.at(want_min, (np.arange(M)[None, :].repeat(N, 0), want[2]), 1)
+        assert np.array_equal(max_count.cpu().numpy(), want_max), tag + " max_count"
+        assert np.array_equal(min_count.cpu().numpy(), want_min), tag + " min_count"
+        assert found[0] == np.sort(np.abs(w.numpy()).ravel())[rank], tag + " selected element"
+        torch.randn(256, 256, device=dev).sum().item()
