@@ -243,8 +243,10 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
     __syncthreads();
     bool fixed = span >= 8;
     int e_lo = 1;
+    bool have_first = false;      // the first item of plane 0 is in the registers (loaded for the window)
     if (fixed) {
         MAM_LOAD_ITEM(0, m_first);
+        have_first = true;
         uint32_t mx = 0u;
         if (row_ok && m_first < M) {
             if (!w_sel) {     // no hand-over: the first trip's weights are gathered for the window as well
@@ -276,7 +278,8 @@ __global__ __launch_bounds__(NT_W) void mam_bwd_x_rows_kernel(
         __syncthreads();
         for (int pl = 0; pl < planes; ++pl) {            // one (argmax, argmin) pair per K range
             int m = m_first;
-            MAM_LOAD_ITEM(pl, m);
+            if (!have_first) MAM_LOAD_ITEM(pl, m);
+            have_first = false;
             for (int t = 0; t < trips; ++t) {
                 const float4 cg = g, c1 = s1, c2 = s2;
                 const int4 a1 = i1, a2 = i2;
