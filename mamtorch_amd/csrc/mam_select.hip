@@ -30,9 +30,11 @@ struct State {
     uint32_t nranks, pad;
     int64_t rank[MAX_RANKS];        // rank still to go within the elements that share the prefix
 };
-// workspace: State, then hist[PASSES][MAX_RANKS][BINS]
+// workspace: State, then hist[PASSES][MAX_RANKS][BINS] of 64-bit counts (the tensors of one selection may hold
+// more than 2^32 elements together; a workgroup's own LDS bins are 32 bits)
+typedef unsigned long long count_t;
 constexpr size_t kHistWords = (size_t)PASSES * MAX_RANKS * BINS;
-constexpr size_t kWorkspaceBytes = 256 + kHistWords * 4;
+constexpr size_t kWorkspaceBytes = 256 + kHistWords * sizeof(count_t);
 
 // keys are 31 bits wide (absolute values: the sign bit is clear): digits of 11, 11 and 9 bits
 __host__ __device__ constexpr int pass_shift(int pass) { return pass == 0 ? 20 : pass == 1 ? 9 : 0; }
@@ -48,9 +50,9 @@ __device__ __forceinline__ uint32_t key_of(float w, const void *aux, const void 
     return (uint32_t)(cnt < 0 ? -cnt : cnt);
 }
 
-__global__ __launch_bounds__(NT) void begin_kernel(State *st, uint32_t *hist, int64_t r0, int64_t r1, int nranks)
+__global__ __launch_bounds__(NT) void begin_kernel(State *st, count_t *hist, int64_t r0, int64_t r1, int nranks)
 {
-    for (size_t i = (size_t)blockIdx.x * NT + threadIdx.x; i < kHistWords; i += (size_t)gridDim.x * NT) hist[i] = 0u;
+    for (size_t i = (size_t)blockIdx.x * NT + threadIdx.x; i < kHistWords; i += (size_t)gridDim.x * NT) hist[i] = 0ull;
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         st->prefix[0] = st->prefix[1] = 0u;
         st->nranks = (uint32_t)nranks;
@@ -64,7 +66,7 @@ __global__ __launch_bounds__(NT) void begin_kernel(State *st, uint32_t *hist, in
 template <int MODE>
 __global__ __launch_bounds__(NT_H) void hist_kernel(const float *__restrict__ w, int64_t ldw, const void *aux,
                                                   const void *aux2, int64_t ld_aux, int64_t M, int64_t K, int vec,
-                                                  const State *__restrict__ st, uint32_t *__restrict__ hist, int pass)
+                                                  const State *__restrict__ st, count_t *__restrict__ hist, int pass)
 {
     __shared__ uint32_t bins[MAX_RANKS][BINS];
     const int tid = threadIdx.x;
@@ -130,15 +132,15 @@ __global__ __launch_bounds__(NT_H) void hist_kernel(const float *__restrict__ w,
     for (int s = 0; s < MAX_RANKS; ++s)
         if (run_count[s]) atomicAdd(&bins[s][run_digit[s]], run_count[s]);
     __syncthreads();
-    uint32_t *out = hist + (size_t)pass * MAX_RANKS * BINS;
+    count_t *out = hist + (size_t)pass * MAX_RANKS * BINS;
     for (int i = tid; i < (one ? 1 : MAX_RANKS) * BINS; i += NT_H) {
         const uint32_t v = (&bins[0][0])[i];
-        if (v) atomicAdd(&out[i], v);
+        if (v) atomicAdd(&out[i], (count_t)v);
     }
 }
 
 // After every tensor has been through pass `pass`: walk the histogram(s) and fix the digit of each rank.
-__global__ __launch_bounds__(NT) void advance_kernel(State *st, const uint32_t *__restrict__ hist, int pass)
+__global__ __launch_bounds__(NT) void advance_kernel(State *st, const count_t *__restrict__ hist, int pass)
 {
     __shared__ int64_t partial[NT];
     const int tid = threadIdx.x;
@@ -149,9 +151,9 @@ __global__ __launch_bounds__(NT) void advance_kernel(State *st, const uint32_t *
     uint32_t digit[MAX_RANKS] = {0u, 0u};
     int64_t rest[MAX_RANKS] = {0, 0};
     for (int s = 0; s < nr; ++s) {
-        const uint32_t *h = hist + ((size_t)pass * MAX_RANKS + (one ? 0 : s)) * BINS;
+        const count_t *h = hist + ((size_t)pass * MAX_RANKS + (one ? 0 : s)) * BINS;
         int64_t sum = 0;
-        for (int b = 0; b < per; ++b) sum += (tid * per + b) < nbins ? h[tid * per + b] : 0u;
+        for (int b = 0; b < per; ++b) sum += (tid * per + b) < nbins ? (int64_t)h[tid * per + b] : 0;
         partial[tid] = sum;
         __syncthreads();
         if (tid == 0) {
@@ -159,7 +161,7 @@ __global__ __launch_bounds__(NT) void advance_kernel(State *st, const uint32_t *
             int t = 0;
             while (t < NT - 1 && below + partial[t] <= r) below += partial[t++];
             int b = t * per;
-            while (b < nbins - 1 && below + h[b] <= r) below += h[b++];
+            while (b < nbins - 1 && below + (int64_t)h[b] <= r) below += (int64_t)h[b++];
             digit[s] = (uint32_t)b;
             rest[s] = r - below;
         }
@@ -179,7 +181,7 @@ __global__ void result_kernel(const State *st, float *out, int as_count)
     if (s < (int)st->nranks) out[s] = as_count ? (float)(int)st->prefix[s] : __uint_as_float(st->prefix[s]);
 }
 
-static uint32_t *hist_of(void *workspace) { return reinterpret_cast<uint32_t *>(static_cast<char *>(workspace) + 256); }
+static count_t *hist_of(void *workspace) { return reinterpret_cast<count_t *>(static_cast<char *>(workspace) + 256); }
 
 }  // namespace selectk
 }  // namespace mam
@@ -225,7 +227,7 @@ extern "C" int mam_select_accumulate(void *workspace, const float *w, int64_t ld
     if (blocks < 1) blocks = 1;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const selectk::State *state = static_cast<const selectk::State *>(workspace);
-    uint32_t *hist = selectk::hist_of(workspace);
+    selectk::count_t *hist = selectk::hist_of(workspace);
 #define MAM_SELECT_LAUNCH(MODE)                                                                                      \
     hipLaunchKernelGGL(selectk::hist_kernel<MODE>, dim3((unsigned)blocks), dim3(selectk::NT_H), 0, st, w, ldw, aux, aux2, \
                        ld_aux, M, K, vec ? 1 : 0, state, hist, pass)
