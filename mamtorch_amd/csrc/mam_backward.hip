@@ -549,8 +549,8 @@ __global__ __launch_bounds__(NT_C) void mam_bwd_w_count_kernel(
 // aligned operands).  A workgroup owns 4 neurons x kc columns in 64-bit fixed-point cells (mam_fixed.h): integer
 // adds are exact and commute, so w_grad does not depend on the order in which the lanes arrive and equals the
 // correctly rounded sum.  An 8-byte cell halves the columns a 64 KiB slab holds, so a neuron quad with K = 4096
-// is covered by two workgroups that each scan the quad's items: 32 against 17 us at 256 x 4096 x 4096, which is
-// why this is an option and not the default.  Terms outside the window (more than ~2^25 below the largest, inf,
+// is covered by two workgroups that each scan the quad's items: 45 against 17 us at 256 x 4096 x 4096 (1.7 to
+// 1.8 times the fp32 kernel's time at batch 12608), which is why this is an option and not the default.  Terms outside the window (more than ~2^25 below the largest, inf,
 // nan) go through the queue and are added in fp64 before the one rounding; if more than QCAP terms of a
 // workgroup fall outside, that workgroup falls back to fp32 LDS atomics (and its cells are then sums in arrival
 // order, within the documented tolerance).
@@ -945,7 +945,9 @@ static int launch_w_count(const float *x, int64_t ldx, const float *grad, const 
                      ((uintptr_t)argmax % 16 == 0) && ((uintptr_t)argmin % 16 == 0) && ((uintptr_t)x_sel % 16 == 0) &&
                      ((uintptr_t)w_grad % 16 == 0) && ((uintptr_t)max_count % 16 == 0) &&
                      ((uintptr_t)min_count % 16 == 0);
-    if (!vec || N >= 2048 || N >= 32768) return 1;
+    // (a count field in LDS is 16 bits wide: at most one pick per batch row and extreme; larger batches go to the
+    // large-batch w_grad route and the count kernel's passes anyway)
+    if (!vec || N >= 2048) return 1;
     const int log2r = 2, R = 4;
     // histogram + count plane of a slab: 4 neurons x kc columns x 8 bytes
     const int64_t lds_cap_bytes = (int64_t)g_lds_floats[dev] * 4;
