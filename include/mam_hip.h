@@ -62,7 +62,8 @@ extern "C" {
 #define MAM_FORWARD_TILING_GROUPS16 2 /* as AUTO, but indices recorded per 16 products at every K   */
 #define MAM_FORWARD_TILING_FUSED_MERGE 3 /* as AUTO, but a K-split call merges inside the forward launch: the
                                             last of a tile's workgroups to finish combines and resolves   */
-#define MAM_BACKWARD_FORK_AUTO (-1) /* from 2^22 outputs on, and under stream capture from 2^16   */
+#define MAM_BACKWARD_FORK_AUTO (-1) /* where it pays: from 2^23 outputs on with at least 1024 neurons (dense),
+                                       2^22 outputs (CSR); under stream capture from 2^16 outputs       */
 #define MAM_BACKWARD_FORK_OFF 0
 #define MAM_BACKWARD_FORK_ON 1
 #define MAM_BACKWARD_ONE_LAUNCH_OFF 0

@@ -1027,7 +1027,12 @@ static int backward_impl(const float *x, int64_t ldx, const float *w, int64_t ld
         if (rc != 1) return rc;
     }
     if (x_grad && w_grad) {
-        ForkedStream fork(st, N * M);
+        // Between eager launches the fork pays from 2^23 outputs on and with at least 1024 neurons, measured with
+        // and without it (us): 12608 x 768 -> 3072 344 / 369, 16384 x 1024 -> 4096 563 / 598, 4096^3 243 / 282,
+        // 8192 x 2048 -> 1024 113 / 121, 16384 x 4096 -> 1024 272 / 282; but 4096 x 1024 -> 1024 62 / 56, and with
+        // 768 neurons (the rows kernel's workgroups are short and mostly waiting, and hold the LDS the w_grad
+        // workgroups need) 12608 x 3072 -> 768 180 / 165, 25216 rows 335 / 316, 8192 rows 116 / 113.
+        ForkedStream fork(st, N * M, N * M >= (1 << 23) && M >= 1024);
         if (fork.forked()) {
             const int rc_x = launch(x_grad, nullptr, fork.side());
             fork.join_later();

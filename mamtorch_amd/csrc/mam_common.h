@@ -45,13 +45,14 @@ int transpose(const float *src, int64_t ld, float *dst, int64_t rows, int64_t co
 //   ForkedStream fork(st, units);      // decides; fork.side() is `st` itself when not forked
 //   launch A on fork.side(); fork.join_later(); launch B on st; rc = fork.join();
 // Between eager launches the two events cost ~15 us, inside a captured graph next to nothing: the fork
-// is taken from 2^22 `units` (outputs of the call) on, and from 2^16 on while `st` is being captured.
+// is taken from 2^22 `units` (outputs of the call) on where the caller says that it pays between eager
+// launches (`eager_pays`), and from 2^16 on while `st` is being captured.
 // Option MAM_OPT_BACKWARD_FORK forces it off / on.  The enqueue sequences of concurrent callers on one
 // device are serialised (the events are reused), so an object of this class holds that device's lock
 // while forked.  The second stream is created by the device's set-up, never inside a capture.
 class ForkedStream {
 public:
-    ForkedStream(hipStream_t st, int64_t units);
+    ForkedStream(hipStream_t st, int64_t units, bool eager_pays = true);
     ~ForkedStream();
     hipStream_t side() const { return side_; }
     bool forked() const { return forked_; }

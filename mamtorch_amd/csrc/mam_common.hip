@@ -219,7 +219,7 @@ int num_cus()
     return cus;
 }
 
-ForkedStream::ForkedStream(hipStream_t st, int64_t units)
+ForkedStream::ForkedStream(hipStream_t st, int64_t units, bool eager_pays)
     : st_(st), side_(st), dev_(-1), forked_(false), recorded_(false)
 {
     if (units <= 0) return;
@@ -230,7 +230,7 @@ ForkedStream::ForkedStream(hipStream_t st, int64_t units)
     } else {
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
         if (st && hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
-        want = units >= (1 << 22) || (capturing == hipStreamCaptureStatusActive && units >= (1 << 16));
+        want = (eager_pays && units >= (1 << 22)) || (capturing == hipStreamCaptureStatusActive && units >= (1 << 16));
     }
     if (!want) return;
     const int dev = ensure_device(st);
